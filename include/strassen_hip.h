@@ -1,0 +1,112 @@
+/* strassen_hip.h -- C ABI of libstrassen_hip.so (gfx950 / MI355X).
+ *
+ * Every entry point takes plain device pointers, sizes and element strides; nothing here
+ * knows about torch.  All work is enqueued on the HIP stream passed in (NULL = the default
+ * stream) and nothing synchronises.  The library never allocates or frees device memory:
+ * the multi-level paths take a caller-provided workspace (sthip_workspace_bytes).
+ *
+ * Return value: 0 on success, a negative sthip_status otherwise; sthip_last_error() then
+ * describes the failure (thread local).
+ *
+ * The reference (vmad18/strassen-triton) is pure Python and has no FFI of its own; each
+ * entry point below names the Python function whose arithmetic it replaces
+ * (paths relative to the reference checkout).
+ */
+#ifndef STRASSEN_HIP_H
+#define STRASSEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define STHIP_VERSION 100
+
+enum sthip_status {
+    STHIP_OK = 0,
+    STHIP_ERR_SHAPE = -1,     /* negative size, mismatched inner dimension, not square where required */
+    STHIP_ERR_DTYPE = -2,     /* unknown dtype / unsupported in-out combination */
+    STHIP_ERR_LAYOUT = -3,    /* an operand has no unit stride, or C is not writable as given */
+    STHIP_ERR_WORKSPACE = -4, /* workspace missing or too small */
+    STHIP_ERR_ARG = -5,       /* null pointer, bad algo / levels */
+    STHIP_ERR_HIP = -6        /* a HIP runtime call failed */
+};
+
+enum sthip_dtype { STHIP_F32 = 0, STHIP_F16 = 1, STHIP_BF16 = 2 };
+
+enum sthip_algo {
+    STHIP_CLASSIC = 0,  /* plain tiled MFMA GEMM (levels is ignored) */
+    STHIP_STRASSEN = 1, /* 7 products, 18 add/sub */
+    STHIP_WINOGRAD = 2  /* 7 products, 15 add/sub (leaf level only; upper levels use Strassen) */
+};
+
+/* General entry: C[b] (+)= A[b] x B[b] for b < batch, A is M x K, B is K x N, C is M x N.
+ * stride*[3] = {batch, row, col} in elements; A and B need one unit stride among (row, col)
+ * each (so NN / NT / TN / TT all work without copies).  in_dtype is the element type of A
+ * and B; out_dtype is that of C and must equal in_dtype or be STHIP_F32.  Products
+ * accumulate in fp32, operand sums are formed in fp32 and rounded once to in_dtype, the
+ * recombination is done in fp32.  levels = 1 runs one fused launch and needs no
+ * workspace; levels >= 2 recurses on the host and needs sthip_workspace_bytes().  Sizes
+ * that are not multiples of 2^levels behave as if zero padded.
+ *
+ * Replaces: _strassen_base (fixed_strassen.py:11-57, fixed_strassen_fp32_agg.py:12-56),
+ * strassen_matmul_n_layers (fixed_strassen.py:59-126, fixed_strassen_fp32_agg.py:58-125),
+ * strassen_matmul_two_layers (strassen.py:742-812) and, with accumulate = 1, the Triton
+ * launchers run_strassen (strassen.py:195-213), run_strassen2 (:674-693),
+ * run_matmul_fp32_accum (:66-88), run_strassen_2_layer_fp32_accum (strassen_2_layer.py:7-15). */
+int sthip_gemm(const void* A, const void* B, void* C,
+               int64_t batch, int64_t M, int64_t N, int64_t K,
+               const int64_t strideA[3], const int64_t strideB[3], const int64_t strideC[3],
+               int in_dtype, int out_dtype, int algo, int levels, int accumulate,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of device workspace sthip_gemm needs for this problem (0 when levels <= 1). */
+size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K,
+                             int in_dtype, int out_dtype, int algo, int levels);
+
+/* C = A x B for square n x n operands, `levels` Strassen levels; B may be a transposed view
+ * (strides in elements).  Replaces strassen_matmul_n_layers(A, B, n_depth, base_dtype)
+ * (fixed_strassen.py:59-126, fixed_strassen_fp32_agg.py:58-125) and, for levels = 1,
+ * _strassen_base (fixed_strassen.py:11-57).  C is contiguous row-major in `dtype`. */
+int sthip_strassen_matmul_n_layers(const void* A, const void* B, void* C, int64_t n,
+                                   int64_t a_row_stride, int64_t a_col_stride,
+                                   int64_t b_row_stride, int64_t b_col_stride,
+                                   int dtype, int levels,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* C += A x B, the contract of the reference's Triton launchers: run_strassen
+ * (strassen.py:195-213; levels = 1), run_strassen2 (strassen.py:674-693; levels = 2),
+ * run_strassen_2_layer_fp32_accum (strassen_2_layer.py:7-15; levels = 2) and
+ * run_matmul_fp32_accum (strassen.py:66-88; algo = STHIP_CLASSIC).  Operands are in
+ * op_dtype (the reference casts tiles to fp16, strassen.py:150-163), C is in c_dtype.
+ * batch = 1 for 2-D inputs.  All tensors contiguous row-major. */
+int sthip_run_accumulate(const void* A, const void* B, void* C,
+                         int64_t batch, int64_t M, int64_t N, int64_t K,
+                         int op_dtype, int c_dtype, int algo, int levels,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* y[rows x D] = x[rows x D] x W^T (+ bias), W is D x D row-major, rows <= D.  The reference
+ * pads x with zero rows up to D x D and slices afterwards (model/layers.py:246-274); here
+ * the missing rows are simply never loaded or stored.  bias may be NULL. */
+int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias, void* y,
+                                  int64_t rows, int64_t D, int dtype, int levels,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* Description of the most recent failure on this thread ("" if none). */
+const char* sthip_last_error(void);
+
+/* STHIP_VERSION the library was built with. */
+int sthip_version(void);
+
+/* Diagnostic: runs the 16-bit transposing LDS read on a 64 x 4 grid of 16-bit values
+ * (value = 4 * lane + element) and writes what each lane received to out[64 * 4] (uint16,
+ * device memory).  Used by the tests to pin the lane mapping the kernels rely on.  No
+ * counterpart in the reference. */
+int sthip_debug_transpose_read(void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STRASSEN_HIP_H */

@@ -1,0 +1,394 @@
+// C-ABI front end of libstrassen_hip.so: argument checking, kernel selection, the host-side
+// recursion for two or more Strassen levels, and the small element-wise kernels that
+// recursion needs.  See include/strassen_hip.h for the contract of every entry point.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/strassen_hip.h"
+#include "sthip_launch.hpp"
+
+namespace sthip {
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+static inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+static inline int elem_size(int dt) { return dt == STHIP_F32 ? 4 : 2; }
+
+// A strided 2-D view of device memory, strides in elements of `dt`.
+struct View {
+    const char* p;
+    int64_t rs, cs;
+};
+
+static const LaunchTable* table_for(int dt, int algo) {
+    switch (dt * 3 + algo) {
+        case 0: return &kLaunch_0_0; case 1: return &kLaunch_0_1; case 2: return &kLaunch_0_2;
+        case 3: return &kLaunch_1_0; case 4: return &kLaunch_1_1; case 5: return &kLaunch_1_2;
+        case 6: return &kLaunch_2_0; case 7: return &kLaunch_2_1; case 8: return &kLaunch_2_2;
+    }
+    return nullptr;
+}
+
+static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// One fused launch: C (+)= A x B with zero or one Strassen / Winograd level.
+// (Mh, Nh, Kh) is the block size used for the split; pass 0 to derive it from the sizes.
+static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
+                        int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
+                        int64_t M, int64_t N, int64_t K, int64_t Mh, int64_t Nh, int64_t Kh,
+                        int dt, bool out_f32, int algo, bool accumulate, hipStream_t stream) {
+    if (M == 0 || N == 0 || batch == 0) return STHIP_OK;
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535)
+        return fail(STHIP_ERR_SHAPE, "size out of range (M=%lld N=%lld K=%lld batch=%lld)",
+                    (long long)M, (long long)N, (long long)K, (long long)batch);
+    if (dt == STHIP_F32 && !out_f32) return fail(STHIP_ERR_DTYPE, "fp32 operands need an fp32 result");
+    const int es = elem_size(dt), epc = 16 / es, bk = 8 * epc;
+    if (algo == STHIP_CLASSIC) { Mh = M; Nh = N; Kh = K; }
+    else {
+        if (Mh <= 0) Mh = ceil_div(M, 2);
+        if (Nh <= 0) Nh = ceil_div(N, 2);
+        if (Kh <= 0) Kh = ceil_div(K, 2);
+    }
+    // operand layouts: contiguous along k, or along m/n
+    const bool a_kc = (A.cs == 1), b_kc = (B.rs == 1);
+    if (!a_kc && A.rs != 1) return fail(STHIP_ERR_LAYOUT, "A has no unit stride (row %lld, col %lld)", (long long)A.rs, (long long)A.cs);
+    if (!b_kc && B.cs != 1) return fail(STHIP_ERR_LAYOUT, "B has no unit stride (row %lld, col %lld)", (long long)B.rs, (long long)B.cs);
+
+    GemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = A.p; p.B = B.p; p.C = C;
+    p.a_rs = A.rs; p.a_cs = A.cs; p.a_bs = a_bs;
+    p.b_rs = B.rs; p.b_cs = B.cs; p.b_bs = b_bs;
+    p.c_rs = c_rs; p.c_cs = c_cs; p.c_bs = c_bs;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.Mh = (int)Mh; p.Nh = (int)Nh; p.Kh = (int)Kh;
+    p.tiles_m = (int)ceil_div(Mh, kBM);
+    p.tiles_n = (int)ceil_div(Nh, kBN);
+    p.out_f32 = out_f32 ? 1 : 0;
+    p.accumulate = accumulate ? 1 : 0;
+    p.group_m = 8;
+
+    // 16-byte loads are legal when the base, the long stride, the batch stride and every
+    // block origin along the contiguous index are multiples of one chunk.
+    const bool split = algo != STHIP_CLASSIC;
+    const int64_t a_long = a_kc ? A.rs : A.cs, b_long = b_kc ? B.cs : B.rs;
+    const int64_t a_blk = a_kc ? Kh : Mh, b_blk = b_kc ? Kh : Nh;
+    p.a_vec = aligned_to(A.p, 16) && a_long % epc == 0 && (batch == 1 || a_bs % epc == 0) && (!split || a_blk % epc == 0);
+    p.b_vec = aligned_to(B.p, 16) && b_long % epc == 0 && (batch == 1 || b_bs % epc == 0) && (!split || b_blk % epc == 0);
+    const size_t c_es = out_f32 ? 4 : es;
+    p.c_vec = c_cs == 1 && aligned_to(C, 4 * c_es) && c_rs % 4 == 0 && (batch == 1 || c_bs % 4 == 0) && (!split || Nh % 4 == 0);
+
+    const bool whole = !split || (M == 2 * Mh && N == 2 * Nh && K == 2 * Kh);
+    const bool fast = whole && Mh % kBM == 0 && Nh % kBN == 0 && Kh % bk == 0 && Kh > 0 && p.a_vec && p.b_vec && p.c_vec;
+
+    const LaunchTable* t = table_for(dt, algo);
+    if (!t) return fail(STHIP_ERR_ARG, "bad dtype/algo (%d, %d)", dt, algo);
+    hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0][fast ? 0 : 1](p, (int)batch, stream);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return STHIP_OK;
+}
+
+// ------------------------------------------------------------------ element-wise kernels
+template <class T> __device__ __forceinline__ float ld_elem(const char* p, int64_t i);
+template <> __device__ __forceinline__ float ld_elem<float>(const char* p, int64_t i) { return reinterpret_cast<const float*>(p)[i]; }
+template <> __device__ __forceinline__ float ld_elem<bf16_t>(const char* p, int64_t i) {
+    return __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(p)[i] << 16);
+}
+template <> __device__ __forceinline__ float ld_elem<f16_t>(const char* p, int64_t i) {
+    return (float)__builtin_bit_cast(_Float16, reinterpret_cast<const uint16_t*>(p)[i]);
+}
+template <class T> __device__ __forceinline__ void st_elem(char* p, int64_t i, float v);
+template <> __device__ __forceinline__ void st_elem<float>(char* p, int64_t i, float v) { reinterpret_cast<float*>(p)[i] = v; }
+template <> __device__ __forceinline__ void st_elem<bf16_t>(char* p, int64_t i, float v) {
+    reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)pack_bf16(v, 0.f);
+}
+template <> __device__ __forceinline__ void st_elem<f16_t>(char* p, int64_t i, float v) {
+    reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)pack_f16(v, 0.f);
+}
+
+// dst[rows x cols] (dense) = X[block a] + sign * X[block b], each block clipped to the
+// logical extent (lim_r, lim_c) of X and read as zero outside it.  sign = 0: copy block a.
+// The sum is formed in fp32 and rounded once (fixed_strassen_fp32_agg.py:87-96).
+template <class T>
+__global__ void block_sum_kernel(char* dst, const char* X, int64_t rs, int64_t cs,
+                                 int ra, int ca, int rb, int cb, int sign,
+                                 int rows, int cols, int lim_r, int lim_c) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)rows * cols) return;
+    const int i = (int)(idx / cols), j = (int)(idx % cols);
+    float v = 0.f;
+    if (ra + i < lim_r && ca + j < lim_c) v = ld_elem<T>(X, (int64_t)(ra + i) * rs + (int64_t)(ca + j) * cs);
+    if (sign != 0 && rb + i < lim_r && cb + j < lim_c) {
+        const float w = ld_elem<T>(X, (int64_t)(rb + i) * rs + (int64_t)(cb + j) * cs);
+        v = sign > 0 ? v + w : v - w;
+    }
+    st_elem<T>(dst, idx, v);
+}
+
+// C blocks from the seven products (dense fp32, mh x nh each):
+// C11 = M1+M4-M5+M7, C12 = M3+M5, C21 = M2+M4, C22 = M1-M2+M3+M6 (fixed_strassen.py:116-119),
+// clipped to M x N, rounded once to the output type.
+template <class TO>
+__global__ void recombine_kernel(char* C, int64_t c_rs, int64_t c_cs, const float* Mbuf, int64_t mstride,
+                                 int mh, int nh, int M, int N, int accumulate) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)mh * nh) return;
+    const int i = (int)(idx / nh), j = (int)(idx % nh);
+    float m[7];
+#pragma unroll
+    for (int q = 0; q < 7; ++q) m[q] = Mbuf[q * mstride + idx];
+    const float c11 = m[0] + m[3] - m[4] + m[6];
+    const float c12 = m[2] + m[4];
+    const float c21 = m[1] + m[3];
+    const float c22 = m[0] - m[1] + m[2] + m[5];
+    const float out[4] = {c11, c12, c21, c22};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int r = i + (q >> 1) * mh, c = j + (q & 1) * nh;
+        if (r >= M || c >= N) continue;
+        const int64_t off = (int64_t)r * c_rs + (int64_t)c * c_cs;
+        float v = out[q];
+        if (accumulate) v += ld_elem<TO>(C, off);
+        st_elem<TO>(C, off, v);
+    }
+}
+
+template <class T>
+__global__ void add_bias_kernel(char* y, const char* bias, int64_t rows, int64_t D) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * D) return;
+    st_elem<T>(y, idx, ld_elem<T>(y, idx) + ld_elem<T>(bias, idx % D));
+}
+
+__global__ void transpose_read_probe_kernel(uint16_t* out) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds[256];
+    const int lane = threadIdx.x;
+    for (int e = 0; e < 4; ++e) lds[lane * 4 + e] = (uint16_t)(lane * 4 + e);
+    __syncthreads();
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(lds + lane * 4));
+    for (int e = 0; e < 4; ++e) out[lane * 4 + e] = (uint16_t)v[e];
+}
+
+static int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "%s launch failed: %s", what, hipGetErrorString(e));
+    return STHIP_OK;
+}
+
+static int block_sum(int dt, char* dst, View X, int ra, int ca, int rb, int cb, int sign,
+                     int64_t rows, int64_t cols, int64_t lim_r, int64_t lim_c, hipStream_t s) {
+    const int64_t n = rows * cols;
+    if (n == 0) return STHIP_OK;
+    const unsigned blocks = (unsigned)ceil_div(n, 256);
+#define GO(T) hipLaunchKernelGGL(block_sum_kernel<T>, dim3(blocks), dim3(256), 0, s, dst, X.p, X.rs, X.cs, ra, ca, rb, cb, sign, (int)rows, (int)cols, (int)lim_r, (int)lim_c)
+    if (dt == STHIP_F32) GO(float); else if (dt == STHIP_F16) GO(f16_t); else GO(bf16_t);
+#undef GO
+    return check_launch("block_sum");
+}
+
+static int recombine(int out_dt, char* C, int64_t c_rs, int64_t c_cs, const float* Mbuf, int64_t mstride,
+                     int64_t mh, int64_t nh, int64_t M, int64_t N, bool accumulate, hipStream_t s) {
+    const int64_t n = mh * nh;
+    if (n == 0) return STHIP_OK;
+    const unsigned blocks = (unsigned)ceil_div(n, 256);
+#define GO(T) hipLaunchKernelGGL(recombine_kernel<T>, dim3(blocks), dim3(256), 0, s, C, c_rs, c_cs, Mbuf, mstride, (int)mh, (int)nh, (int)M, (int)N, accumulate ? 1 : 0)
+    if (out_dt == STHIP_F32) GO(float); else if (out_dt == STHIP_F16) GO(f16_t); else GO(bf16_t);
+#undef GO
+    return check_launch("recombine");
+}
+
+// Strassen product table in the reference's numbering (fixed_strassen.py:88-114):
+// {A block a, A block b, sign} x {B block a, B block b, sign}; block ids 0=11 1=12 2=21 3=22,
+// sign 0 = single block.
+struct Term { int a, b, sign; };
+static const Term kATerms[7] = {{0, 3, +1}, {2, 3, +1}, {0, 0, 0}, {3, 0, 0}, {0, 1, +1}, {2, 0, -1}, {1, 3, -1}};
+static const Term kBTerms[7] = {{0, 3, +1}, {0, 0, 0}, {1, 3, -1}, {2, 0, -1}, {3, 0, 0}, {0, 1, +1}, {2, 3, +1}};
+
+static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels) {
+    if (levels <= 1) return 0;
+    const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
+    const size_t es = elem_size(dt);
+    return align256(mh * kh * es) + align256(kh * nh * es) + 7 * align256(mh * nh * 4) +
+           workspace_for(mh, nh, kh, dt, levels - 1);
+}
+
+// C (+)= A x B with `levels` levels.  (Mp, Np, Kp) >= (M, N, K) are the padded sizes the
+// split is taken on (multiples of 2^levels); everything outside (M, N, K) reads as zero.
+static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
+                    int64_t M, int64_t N, int64_t K, int64_t Mp, int64_t Np, int64_t Kp,
+                    int dt, int out_dt, int algo, int levels, bool accumulate,
+                    char* ws, size_t ws_bytes, hipStream_t stream) {
+    const bool out_f32 = out_dt == STHIP_F32;
+    if (algo == STHIP_CLASSIC || levels <= 0)
+        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, 0, 0, 0, dt, out_f32, STHIP_CLASSIC, accumulate, stream);
+    const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
+    if (levels == 1)
+        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, mh, nh, kh, dt, out_f32, algo, accumulate, stream);
+
+    const size_t es = elem_size(dt);
+    const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es), m_b = align256(mh * nh * 4);
+    const size_t need = sa_b + sb_b + 7 * m_b;
+    if (!ws || ws_bytes < need) return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, need);
+    char* SA = ws;
+    char* SB = ws + sa_b;
+    char* Mbuf = ws + sa_b + sb_b;
+    char* child_ws = ws + need;
+    const size_t child_bytes = ws_bytes - need;
+
+    for (int q = 0; q < 7; ++q) {
+        const Term ta = kATerms[q], tb = kBTerms[q];
+        View a, b;
+        int64_t am = mh, ak = kh, bk = kh, bn = nh;   // logical extents of the operands handed down
+        // A operand: a single block that lies fully inside A is used in place
+        const int ara = (ta.a >> 1) * (int)mh, aca = (ta.a & 1) * (int)kh;
+        if (ta.sign == 0 && ara + mh <= M && aca + kh <= K) {
+            a = {A.p + ((int64_t)ara * A.rs + (int64_t)aca * A.cs) * (int64_t)es, A.rs, A.cs};
+        } else {
+            int rc = block_sum(dt, SA, A, ara, aca, (ta.b >> 1) * (int)mh, (ta.b & 1) * (int)kh, ta.sign, mh, kh, M, K, stream);
+            if (rc) return rc;
+            a = {SA, kh, 1};
+        }
+        const int bra = (tb.a >> 1) * (int)kh, bca = (tb.a & 1) * (int)nh;
+        if (tb.sign == 0 && bra + kh <= K && bca + nh <= N) {
+            b = {B.p + ((int64_t)bra * B.rs + (int64_t)bca * B.cs) * (int64_t)es, B.rs, B.cs};
+        } else {
+            int rc = block_sum(dt, SB, B, bra, bca, (tb.b >> 1) * (int)kh, (tb.b & 1) * (int)nh, tb.sign, kh, nh, K, N, stream);
+            if (rc) return rc;
+            b = {SB, nh, 1};
+        }
+        int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, am, bn, ak, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
+                          false, child_ws, child_bytes, stream);
+        (void)bk;
+        if (rc) return rc;
+    }
+    return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, stream);
+}
+
+static int check_common(const void* A, const void* B, const void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                        int in_dt, int out_dt, int algo, int levels) {
+    if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(STHIP_ERR_SHAPE, "negative size");
+    if (in_dt < 0 || in_dt > 2 || out_dt < 0 || out_dt > 2) return fail(STHIP_ERR_DTYPE, "unknown dtype (%d, %d)", in_dt, out_dt);
+    if (out_dt != in_dt && out_dt != STHIP_F32) return fail(STHIP_ERR_DTYPE, "out dtype must equal in dtype or be fp32");
+    if (algo < 0 || algo > 2) return fail(STHIP_ERR_ARG, "unknown algo %d", algo);
+    if (levels < 0 || levels > 8) return fail(STHIP_ERR_ARG, "levels must be in [0, 8], got %d", levels);
+    if (batch > 0 && M > 0 && N > 0 && (!C || (K > 0 && (!A || !B)))) return fail(STHIP_ERR_ARG, "null pointer");
+    return STHIP_OK;
+}
+
+}  // namespace sthip
+
+using namespace sthip;
+
+extern "C" {
+
+int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+               const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
+               int in_dtype, int out_dtype, int algo, int levels, int accumulate,
+               void* workspace, size_t workspace_bytes, void* stream) {
+    g_err[0] = 0;
+    int rc = check_common(A, B, C, batch, M, N, K, in_dtype, out_dtype, algo, levels);
+    if (rc) return rc;
+    if (!sA || !sB || !sC) return fail(STHIP_ERR_ARG, "null stride array");
+    if (batch == 0 || M == 0 || N == 0) return STHIP_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int es = elem_size(in_dtype), ces = elem_size(out_dtype);
+    if (algo == STHIP_CLASSIC) levels = 0;
+    if (algo != STHIP_CLASSIC && levels == 0) algo = STHIP_CLASSIC;
+    const int64_t q = (int64_t)1 << levels;
+    const int64_t Mp = round_up(M, q), Np = round_up(N, q), Kp = round_up(K, q);
+    if (levels <= 1) {
+        View a = {reinterpret_cast<const char*>(A), sA[1], sA[2]};
+        View b = {reinterpret_cast<const char*>(B), sB[1], sB[2]};
+        return launch_fused(a, b, reinterpret_cast<char*>(C), sC[1], sC[2], batch, sA[0], sB[0], sC[0], M, N, K,
+                            Mp / 2, Np / 2, Kp / 2, in_dtype, out_dtype == STHIP_F32, algo, accumulate != 0, s);
+    }
+    for (int64_t bi = 0; bi < batch; ++bi) {
+        View a = {reinterpret_cast<const char*>(A) + bi * sA[0] * es, sA[1], sA[2]};
+        View b = {reinterpret_cast<const char*>(B) + bi * sB[0] * es, sB[1], sB[2]};
+        char* c = reinterpret_cast<char*>(C) + bi * sC[0] * ces;
+        rc = multiply(a, b, c, sC[1], sC[2], M, N, K, Mp, Np, Kp, in_dtype, out_dtype, algo, levels, accumulate != 0,
+                      reinterpret_cast<char*>(workspace), workspace_bytes, s);
+        if (rc) return rc;
+    }
+    return STHIP_OK;
+}
+
+size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {
+    (void)batch; (void)out_dtype;
+    if (algo == STHIP_CLASSIC || levels <= 1 || M <= 0 || N <= 0 || K < 0 || levels > 8 || in_dtype < 0 || in_dtype > 2) return 0;
+    const int64_t q = (int64_t)1 << levels;
+    return workspace_for(round_up(M, q), round_up(N, q), round_up(K, q), in_dtype, levels);
+}
+
+int sthip_strassen_matmul_n_layers(const void* A, const void* B, void* C, int64_t n,
+                                   int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs,
+                                   int dtype, int levels, void* workspace, size_t workspace_bytes, void* stream) {
+    const int64_t sA[3] = {0, a_rs, a_cs}, sB[3] = {0, b_rs, b_cs}, sC[3] = {0, n, 1};
+    if (levels < 1) return fail(STHIP_ERR_ARG, "levels must be >= 1, got %d", levels);
+    return sthip_gemm(A, B, C, 1, n, n, n, sA, sB, sC, dtype, dtype, STHIP_STRASSEN, levels, 0, workspace, workspace_bytes, stream);
+}
+
+int sthip_run_accumulate(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                         int op_dtype, int c_dtype, int algo, int levels,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    const int64_t sA[3] = {M * K, K, 1}, sB[3] = {K * N, N, 1}, sC[3] = {M * N, N, 1};
+    return sthip_gemm(A, B, C, batch, M, N, K, sA, sB, sC, op_dtype, c_dtype, algo, levels, 1, workspace, workspace_bytes, stream);
+}
+
+int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias, void* y,
+                                  int64_t rows, int64_t D, int dtype, int levels,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    g_err[0] = 0;
+    int rc = check_common(x, W, y, 1, rows, D, D, dtype, dtype, STHIP_STRASSEN, levels);
+    if (rc) return rc;
+    if (levels < 1) return fail(STHIP_ERR_ARG, "levels must be >= 1, got %d", levels);
+    if (rows > D) return fail(STHIP_ERR_SHAPE, "rows (%lld) > D (%lld): the input cannot be padded to D x D", (long long)rows, (long long)D);
+    if (rows == 0 || D == 0) return STHIP_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    // The reference pads x to D x D (model/layers.py:261-262): split on the padded size.
+    const int64_t q = (int64_t)1 << levels;
+    const int64_t Dp = round_up(D, q);
+    View a = {reinterpret_cast<const char*>(x), D, 1};
+    View b = {reinterpret_cast<const char*>(W), 1, D};   // W^T as a view
+    rc = multiply(a, b, reinterpret_cast<char*>(y), D, 1, rows, D, D, Dp, Dp, Dp, dtype, dtype, STHIP_STRASSEN, levels, false,
+                  reinterpret_cast<char*>(workspace), workspace_bytes, s);
+    if (rc) return rc;
+    if (bias) {
+        const int64_t n = rows * D;
+        const unsigned blocks = (unsigned)ceil_div(n, 256);
+        char* yy = reinterpret_cast<char*>(y);
+        const char* bb = reinterpret_cast<const char*>(bias);
+        if (dtype == STHIP_F32) hipLaunchKernelGGL(add_bias_kernel<float>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
+        else if (dtype == STHIP_F16) hipLaunchKernelGGL(add_bias_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
+        else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
+        return check_launch("add_bias");
+    }
+    return STHIP_OK;
+}
+
+const char* sthip_last_error(void) { return g_err; }
+
+int sthip_version(void) { return STHIP_VERSION; }
+
+int sthip_debug_transpose_read(void* out, void* stream) {
+    g_err[0] = 0;
+    if (!out) return fail(STHIP_ERR_ARG, "null pointer");
+    hipLaunchKernelGGL(transpose_read_probe_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream),
+                       reinterpret_cast<uint16_t*>(out));
+    return check_launch("transpose_read_probe");
+}
+
+}  // extern "C"

@@ -1,0 +1,39 @@
+// Launch table shared by the kernel instantiation units and the C-ABI front end.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "sthip_kernel.hpp"
+
+namespace sthip {
+
+enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+
+// One table per (element type, algorithm), indexed [a_kc][b_kc][edge]; each is defined by
+// one compilation of sthip_inst.hip.
+typedef hipError_t (*LaunchFn)(const GemmParams&, int batch, hipStream_t);
+struct LaunchTable { LaunchFn fn[2][2][2]; };
+#define STHIP_DECLARE_TABLE(T, A) extern const LaunchTable kLaunch_##T##_##A;
+STHIP_DECLARE_TABLE(0, 0) STHIP_DECLARE_TABLE(0, 1) STHIP_DECLARE_TABLE(0, 2)
+STHIP_DECLARE_TABLE(1, 0) STHIP_DECLARE_TABLE(1, 1) STHIP_DECLARE_TABLE(1, 2)
+STHIP_DECLARE_TABLE(2, 0) STHIP_DECLARE_TABLE(2, 1) STHIP_DECLARE_TABLE(2, 2)
+#undef STHIP_DECLARE_TABLE
+
+template <class T, int ALGO, bool A_KC, bool B_KC, bool EDGE>
+hipError_t launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
+    using C = Ctx<T, A_KC, B_KC>;
+    auto kern = gemm_kernel<T, ALGO, A_KC, B_KC, EDGE>;
+    // More than 64 KiB of dynamic LDS needs an explicit opt-in, once per device.
+    static bool opted[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && !opted[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES);
+        if (e != hipSuccess) return e;
+        opted[dev] = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads), C::SMEM_BYTES, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace sthip

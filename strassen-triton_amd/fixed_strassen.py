@@ -1,0 +1,86 @@
+"""Drop-in for the reference's fixed_strassen.py on MI355X.
+
+Same names and call signatures (`_strassen_base`, `strassen_matmul_n_layers`,
+`LinearStrassen`), but the quadrant sums, the seven products and the recombination run in
+one hand-written HIP kernel per level instead of torch ops under torch.compile.  Tensors
+must be on the GPU.
+"""
+from __future__ import annotations
+
+from math import log2
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+import strassen_hip
+from _levels import LEAF, practical_levels, reference_levels
+
+
+def _check_square(A: Tensor, B: Tensor) -> int:
+    if A.dim() != 2 or B.dim() != 2 or A.shape[0] != A.shape[1] or tuple(A.shape) != tuple(B.shape):
+        raise ValueError("Input matrices must be square and have the same dimensions.")
+    return A.shape[0]
+
+
+def _strassen_base(A: Tensor, B: Tensor, base_dtype=torch.float32) -> Tensor:
+    """One Strassen level (reference fixed_strassen.py:11-57); base_dtype is ignored here as
+    it is there.  Inputs of 16 rows or fewer are multiplied classically (:20-21)."""
+    n = _check_square(A, B)
+    if n <= LEAF:
+        return strassen_hip.matmul(A, B, algo="classic", levels=0)
+    return strassen_hip.matmul(A, B, algo="strassen", levels=1)
+
+
+def strassen_matmul_n_layers(A: Tensor, B: Tensor, n_depth: int = 2, base_dtype=torch.float32) -> Tensor:
+    """n_depth-level Strassen product (reference fixed_strassen.py:59-126)."""
+    n = _check_square(A, B)
+    levels = practical_levels(n, reference_levels(n, n_depth))
+    if levels == 0:
+        return strassen_hip.matmul(A, B, algo="classic", levels=0)
+    return strassen_hip.matmul(A, B, algo="strassen", levels=levels)
+
+
+class _LinearFn(torch.autograd.Function):
+    """y = x W^T + b with the forward in one C-ABI call; dgrad dX = dY W and wgrad
+    dW = dY^T X are Strassen products over views of the saved tensors."""
+
+    @staticmethod
+    def forward(ctx, x2d, weight, bias, levels):
+        ctx.save_for_backward(x2d, weight)
+        ctx.levels, ctx.has_bias = levels, bias is not None
+        return strassen_hip.linear_forward(x2d, weight, bias, levels)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2d, weight = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = strassen_hip.gemm(dy, weight, levels=1) if ctx.needs_input_grad[0] else None
+        dw = strassen_hip.gemm(dy.t(), x2d, levels=1) if ctx.needs_input_grad[1] else None
+        db = dy.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return dx, dw, db, None
+
+
+class LinearStrassen(nn.Linear):
+    """nn.Linear whose matmul is the Strassen kernel (reference fixed_strassen.py:128-169,
+    model/layers.py:232-274): square power-of-two features, at most D input rows."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=torch.float32,
+                 depth: int = 1, device: str = "cuda") -> None:
+        assert in_features == out_features and (log2(in_features)).is_integer(), \
+            "Transform must be square and a power of 2"
+        super().__init__(in_features, out_features, bias, device, dtype)
+        self.depth = depth
+
+    def forward(self, input: Tensor):
+        *batch_dims, D_in = input.shape
+        assert D_in == self.in_features, "Input dim mismatch"
+        D = self.in_features
+        M = input.numel() // D
+        if M > D:
+            raise ValueError(
+                f"Input M ({M}) > D ({D}). Cannot pad input to DxD. "
+                f"You MUST use the method that pads BOTH input and weights to PxP.")
+        levels = max(1, practical_levels(D, reference_levels(D, self.depth)))
+        out = _LinearFn.apply(input.reshape(M, D), self.weight, self.bias, levels)
+        return out.view(*batch_dims, D)

@@ -1,0 +1,6 @@
+"""Host side of the MI355X Strassen library: tensors in, C-ABI calls out."""
+from .ops import (ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD, StrassenMatmul, gemm, linear_forward,
+                  matmul, run_accumulate)
+
+__all__ = ["gemm", "matmul", "run_accumulate", "linear_forward", "StrassenMatmul",
+           "ALGO_CLASSIC", "ALGO_STRASSEN", "ALGO_WINOGRAD"]

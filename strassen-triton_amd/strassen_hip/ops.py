@@ -1,0 +1,160 @@
+"""torch.Tensor front end of the C ABI.
+
+PyTorch is used for device memory and streams only; all arithmetic happens in the HIP
+kernels behind libstrassen_hip.so.  Tensors must live on the GPU: there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _capi
+
+ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD = 0, 1, 2
+_ALGOS = {"classic": ALGO_CLASSIC, "strassen": ALGO_STRASSEN, "winograd": ALGO_WINOGRAD}
+_DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "strassen_hip runs on MI355X tensors only (got a tensor on "
+                f"{t.device}); there is no CPU implementation in this library")
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dt}; use float32, float16 or bfloat16") from None
+
+
+def _unit_stride(t: torch.Tensor) -> torch.Tensor:
+    """The kernels read any matrix with a unit stride along rows or columns."""
+    if t.stride(-1) == 1 or t.stride(-2) == 1:
+        return t
+    return t.contiguous()
+
+
+def _strides3(t: torch.Tensor):
+    if t.dim() == 2:
+        s = (0, t.stride(0), t.stride(1))
+    else:
+        s = (t.stride(0) if t.shape[0] > 1 else 0, t.stride(1), t.stride(2))
+    return (ctypes.c_int64 * 3)(*s)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _workspace(nbytes: int, device) -> tuple[torch.Tensor | None, int]:
+    if nbytes == 0:
+        return None, 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr()
+
+
+def gemm(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor | None = None, *, algo="strassen",
+         levels: int = 1, accumulate: bool = False, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """out (+)= A @ B through sthip_gemm.  A: (b,) M x K, B: (b,) K x N, same dtype."""
+    _require_gpu(A, B)
+    lib = _capi.load()
+    algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    if A.dim() != B.dim() or A.dim() not in (2, 3):
+        raise ValueError(f"expected two 2-D or two 3-D tensors, got {tuple(A.shape)} and {tuple(B.shape)}")
+    if A.dtype != B.dtype:
+        raise TypeError(f"operand dtypes differ: {A.dtype} vs {B.dtype}")
+    if A.shape[-1] != B.shape[-2] or (A.dim() == 3 and A.shape[0] != B.shape[0]):
+        raise ValueError(f"shape mismatch: {tuple(A.shape)} @ {tuple(B.shape)}")
+    batch = A.shape[0] if A.dim() == 3 else 1
+    M, K, N = A.shape[-2], A.shape[-1], B.shape[-1]
+    in_dt = _dtype_code(A.dtype)
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate=True needs an `out` tensor")
+        out = torch.empty(A.shape[:-1] + (N,), dtype=out_dtype or A.dtype, device=A.device)
+    else:
+        _require_gpu(out)
+        if tuple(out.shape) != tuple(A.shape[:-1]) + (N,):
+            raise ValueError(f"out has shape {tuple(out.shape)}, expected {tuple(A.shape[:-1]) + (N,)}")
+    out_dt = _dtype_code(out.dtype)
+    A, B = _unit_stride(A), _unit_stride(B)
+    nbytes = lib.sthip_workspace_bytes(batch, M, N, K, in_dt, out_dt, algo, levels)
+    ws, ws_ptr = _workspace(nbytes, A.device)
+    with torch.cuda.device(A.device):
+        _capi.check(lib.sthip_gemm(A.data_ptr(), B.data_ptr(), out.data_ptr(), batch, M, N, K,
+                                   _strides3(A), _strides3(B), _strides3(out), in_dt, out_dt, algo, levels,
+                                   1 if accumulate else 0, ws_ptr, nbytes, _stream()))
+    return out
+
+
+class StrassenMatmul(torch.autograd.Function):
+    """A @ B with gradients that are Strassen products themselves:
+    dA = dC @ B^T and dB = A^T @ dC read the saved operands through transposed views."""
+
+    @staticmethod
+    def forward(ctx, A, B, algo, levels):
+        ctx.save_for_backward(A, B)
+        ctx.algo, ctx.levels = algo, levels
+        return gemm(A, B, algo=algo, levels=levels)
+
+    @staticmethod
+    def backward(ctx, dC):
+        A, B = ctx.saved_tensors
+        dC = dC.contiguous()
+        dA = gemm(dC, B.transpose(-1, -2), algo=ctx.algo, levels=ctx.levels) if ctx.needs_input_grad[0] else None
+        dB = gemm(A.transpose(-1, -2), dC, algo=ctx.algo, levels=ctx.levels) if ctx.needs_input_grad[1] else None
+        return dA, dB, None, None
+
+
+def matmul(A: torch.Tensor, B: torch.Tensor, algo="strassen", levels: int = 1) -> torch.Tensor:
+    """Differentiable A @ B."""
+    if torch.is_grad_enabled() and (A.requires_grad or B.requires_grad):
+        return StrassenMatmul.apply(A, B, algo, levels)
+    return gemm(A, B, algo=algo, levels=levels)
+
+
+def run_accumulate(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, *, algo="strassen", levels: int = 1,
+                   operand_dtype: torch.dtype | None = torch.float16) -> None:
+    """C += A @ B in place (sthip_run_accumulate).  Operands are cast to operand_dtype first
+    when given, as the reference's Triton kernels cast every tile they load."""
+    _require_gpu(A, B, C)
+    lib = _capi.load()
+    algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    if operand_dtype is not None:
+        A, B = A.to(operand_dtype), B.to(operand_dtype)
+    A, B = A.contiguous(), B.contiguous()
+    batch = A.shape[0] if A.dim() == 3 else 1
+    M, K, N = A.shape[-2], A.shape[-1], B.shape[-1]
+    op_dt = _dtype_code(A.dtype)
+    target = C
+    if not C.is_contiguous() or (C.dtype != A.dtype and C.dtype != torch.float32):
+        target = C.to(torch.float32).contiguous()
+    c_dt = _dtype_code(target.dtype)
+    nbytes = lib.sthip_workspace_bytes(batch, M, N, K, op_dt, c_dt, algo, levels)
+    ws, ws_ptr = _workspace(nbytes, A.device)
+    with torch.cuda.device(A.device):
+        _capi.check(lib.sthip_run_accumulate(A.data_ptr(), B.data_ptr(), target.data_ptr(), batch, M, N, K,
+                                             op_dt, c_dt, algo, levels, ws_ptr, nbytes, _stream()))
+    if target is not C:
+        C.copy_(target)
+
+
+def linear_forward(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, levels: int) -> torch.Tensor:
+    """y = x2d @ weight.T (+ bias) for a square weight (sthip_linear_strassen_forward)."""
+    _require_gpu(x2d, weight)
+    lib = _capi.load()
+    rows, D = x2d.shape
+    x2d, weight = x2d.contiguous(), weight.contiguous()
+    dt = _dtype_code(x2d.dtype)
+    y = torch.empty((rows, D), dtype=x2d.dtype, device=x2d.device)
+    nbytes = lib.sthip_workspace_bytes(1, D, D, D, dt, dt, ALGO_STRASSEN, levels)
+    ws, ws_ptr = _workspace(nbytes, x2d.device)
+    b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
+    with torch.cuda.device(x2d.device):
+        _capi.check(lib.sthip_linear_strassen_forward(x2d.data_ptr(), weight.data_ptr(), b_ptr, y.data_ptr(),
+                                                      rows, D, dt, levels, ws_ptr, nbytes, _stream()))
+    return y

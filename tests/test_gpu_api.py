@@ -1,0 +1,123 @@
+"""GPU tests of the reference-shaped call surface: same names, arguments, return values
+and exceptions as strassen.py / fixed_strassen*.py / strassen_2_layer.py / model/layers.py."""
+import pytest
+import torch
+
+from oracle import strassen_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _ints(shape, seed, lo=-1, hi=1, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, shape, generator=g).to(dtype)
+
+
+def test_run_launchers_accumulate_in_place():
+    """run_*: C += A @ B, return None (reference strassen.py:184-192; smoke of :815-825 uses
+    512 x 512 fp32 with C = zeros)."""
+    import strassen
+    import strassen_2_layer
+    torch.manual_seed(1234)
+    a, b = torch.randn(512, 512), torch.randn(512, 512)
+    for fn, cast in ((strassen.run_strassen, torch.float16), (strassen.run_strassen2, torch.float16),
+                     (strassen.run_matmul_fp32_accum, None), (strassen_2_layer.run_strassen_2_layer_fp32_accum, None)):
+        c0 = torch.randn(512, 512)
+        c = c0.clone().cuda()
+        assert fn(a.cuda(), b.cuda(), c) is None
+        want = O.tile_kernel_semantics(a, b, c0, cast)
+        tol = 2e-2 if cast is not None else 1e-5
+        assert O.rel_fro(c.cpu(), want) <= tol, fn.__name__
+    # batched, fp16 C, exact integers
+    A, B = _ints((2, 128, 64), 1, dtype=torch.float16), _ints((2, 64, 256), 2, dtype=torch.float16)
+    C0 = _ints((2, 128, 256), 3, -3, 3, torch.float16)
+    C = C0.clone().cuda()
+    strassen.run_strassen(A.cuda(), B.cuda(), C)
+    assert torch.equal(C.cpu().double(), C0.double() + A.double() @ B.double())
+    with pytest.raises(AssertionError):
+        strassen.run_strassen(torch.zeros(4, 5).cuda(), torch.zeros(6, 4).cuda(), torch.zeros(4, 4).cuda())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,depth", [(16, 1), (64, 1), (256, 2), (256, 3), (512, 2), (64, 7)])
+def test_matrix_level_functions(dtype, n, depth):
+    import fixed_strassen as fs
+    import fixed_strassen_fp32_agg as agg
+    import strassen
+    assert agg.agg_dtype == torch.float32
+    A, B = _ints((n, n), 5, dtype=dtype), _ints((n, n), 6, dtype=dtype)
+    want = A.double() @ B.double()
+    outs = [fs.strassen_matmul_n_layers(A.cuda(), B.cuda(), depth),
+            agg.strassen_matmul_n_layers(A.cuda(), B.cuda(), depth, dtype)]
+    if depth == 1:
+        outs += [fs._strassen_base(A.cuda(), B.cuda()), agg._strassen_base(A.cuda(), B.cuda(), dtype),
+                 strassen._strassen_base(A.cuda(), B.cuda())]
+    if depth == 2:
+        outs.append(strassen.strassen_matmul_two_layers(A.cuda(), B.cuda()))
+    for C in outs:
+        assert C.dtype == dtype and C.shape == (n, n)
+        if want.abs().max() <= 128:
+            assert torch.equal(C.cpu().double(), want)
+        else:
+            assert O.rel_fro(C.cpu(), want) <= 2e-2
+
+
+def test_two_layers_validation():
+    import strassen
+    with pytest.raises(ValueError, match="square"):
+        strassen.strassen_matmul_two_layers(torch.zeros(8, 4).cuda(), torch.zeros(4, 8).cuda())
+    with pytest.raises(ValueError, match="divisible by 4"):
+        strassen.strassen_matmul_two_layers(torch.zeros(6, 6).cuda(), torch.zeros(6, 6).cuda())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("depth", [1, 2])
+def test_linear_strassen_forward_backward(dtype, depth):
+    from model.layers import LinearStrassen
+    D = 256
+    lin = LinearStrassen(D, D, bias=True, dtype=dtype, depth=depth, device="cuda")
+    with torch.no_grad():
+        lin.weight.copy_(_ints((D, D), 7).to(dtype))
+        lin.bias.copy_(_ints((D,), 8).to(dtype))
+    x = _ints((3, 40, D), 9).to(dtype)
+    y = lin(x.cuda())
+    want = O.linear_strassen_forward(x.float(), lin.weight.detach().cpu().float(), lin.bias.detach().cpu().float(), depth)
+    assert y.shape == (3, 40, D) and y.dtype == dtype
+    if want.abs().max() <= 128:
+        assert torch.equal(y.detach().cpu().float(), want)
+    else:
+        assert O.rel_fro(y.detach().cpu(), want) <= 2e-2
+    # gradients against plain autograd on the same integers
+    xg = x.cuda().requires_grad_()
+    g = _ints((3, 40, D), 10).to(dtype).cuda()
+    lin.zero_grad()
+    lin(xg).backward(g)
+    xr = x.float().requires_grad_()
+    Wr = lin.weight.detach().cpu().float().requires_grad_()
+    br = lin.bias.detach().cpu().float().requires_grad_()
+    (xr @ Wr.T + br).backward(g.cpu().float())
+    for got, ref in ((xg.grad, xr.grad), (lin.weight.grad, Wr.grad), (lin.bias.grad, br.grad)):
+        assert O.rel_fro(got.cpu(), ref) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    with pytest.raises(ValueError, match="Cannot pad input"):
+        lin(torch.zeros(D + 1, D, dtype=dtype, device="cuda"))
+    with pytest.raises(AssertionError, match="square and a power of 2"):
+        LinearStrassen(96, 96, device="cuda")
+
+
+def test_replace_linear_with_strassen(capsys):
+    import torch.nn as nn
+    from model.layers import LinearStrassen, replace_linear_with_strassen
+    net = nn.Sequential(nn.Linear(256, 256), nn.ReLU(), nn.Sequential(nn.Linear(256, 64), nn.Linear(64, 64))).cuda()
+    x = torch.randn(32, 256, device="cuda")
+    before = net(x)
+    replace_linear_with_strassen(net, min_size=128, depth=1)
+    out = capsys.readouterr().out
+    assert "Replacing '0' with LinearStrassen." in out and "Skipping" in out
+    assert isinstance(net[0], LinearStrassen) and not isinstance(net[2][0], LinearStrassen)
+    assert O.rel_fro(net(x).cpu(), before.cpu()) <= 1e-5
+
+
+def test_cpu_tensors_are_refused():
+    import fixed_strassen
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        fixed_strassen._strassen_base(torch.zeros(32, 32), torch.zeros(32, 32))

@@ -1,0 +1,228 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle.
+
+Bit-exact where arithmetic is exact (small-integer inputs: every operand sum, product and
+partial sum is an integer that fp32 -- and, where stated, bf16/fp16 -- holds exactly), and
+within the stated relative Frobenius tolerance on seeded Gaussian inputs:
+    fp32            <= 1e-5
+    bf16 / fp16     <= 2e-2   (fp32 accumulation and aggregation)
+"""
+import os
+
+import pytest
+import torch
+
+from oracle import strassen_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import strassen_hip
+    from strassen_hip import _capi
+    _capi.load()
+    return strassen_hip
+
+
+def _ints(shape, seed, lo=-2, hi=2, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, shape, generator=g).to(dtype)
+
+
+def _gauss(shape, seed, scale, dtype):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _layout(X, transposed):
+    """Same values; `transposed` stores the matrix column-major (a .T view of a contiguous tensor)."""
+    Xg = X.cuda()
+    if transposed:
+        return Xg.transpose(-1, -2).contiguous().transpose(-1, -2)
+    return Xg
+
+
+def test_transpose_read_lane_mapping(hip):
+    """Lane i of a 16-lane group receives column i of the 4 x 16 block the group addressed."""
+    from strassen_hip import _capi
+    out = torch.zeros(256, dtype=torch.int16, device="cuda")
+    _capi.check(_capi.load().sthip_debug_transpose_read(out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    got = out.cpu().view(64, 4).tolist()
+    for lane in range(64):
+        grp, i = lane // 16, lane % 16
+        for e in range(4):
+            src_lane = grp * 16 + 4 * e + i // 4
+            assert got[lane][e] == 4 * src_lane + i % 4, (lane, e, got[lane])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (512, 256, 384), (200, 136, 72), (33, 17, 65), (1, 5, 3), (130, 258, 2)])
+def test_integer_kat_exact(hip, dtype, algo, ta, tb, shape):
+    """Entries in [-2, 2]: the fp32 result must equal the fp64 classical product bit for bit."""
+    M, N, K = shape
+    A, B = _ints((M, K), 1, dtype=dtype), _ints((K, N), 2, dtype=dtype)
+    want = A.double() @ B.double()
+    C = hip.gemm(_layout(A, ta), _layout(B, tb), algo=algo, levels=1, out_dtype=torch.float32)
+    assert torch.equal(C.cpu().double(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (96, 40, 100)])
+def test_integer_kat_exact_native_output(hip, dtype, algo, shape):
+    """Entries in {-1, 0, 1}, K <= 128: |C| <= 128 is exact in bf16 and fp16 too."""
+    M, N, K = shape
+    A, B = _ints((M, K), 3, -1, 1, dtype), _ints((K, N), 4, -1, 1, dtype)
+    C = hip.gemm(A.cuda(), B.cuda(), algo=algo, levels=1)
+    assert C.dtype == dtype
+    assert torch.equal(C.cpu().double(), A.double() @ B.double())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("levels,shape", [(2, (512, 512, 512)), (2, (300, 260, 200)), (3, (512, 512, 512)), (2, (67, 35, 129))])
+def test_integer_kat_multi_level(hip, dtype, levels, shape):
+    M, N, K = shape
+    A, B = _ints((M, K), 5, -1, 1, dtype), _ints((K, N), 6, -1, 1, dtype)
+    C = hip.gemm(A.cuda(), B.cuda(), algo="strassen", levels=levels, out_dtype=torch.float32)
+    assert torch.equal(C.cpu().double(), A.double() @ B.double())
+
+
+@pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
+def test_structured_inputs(hip, algo):
+    n = 256
+    X = _ints((n, n), 11)
+    I = torch.eye(n)
+    f = lambda a, b: hip.gemm(a.cuda(), b.cuda(), algo=algo).cpu()
+    assert torch.equal(f(X, I), X) and torch.equal(f(I, X), X)
+    assert torch.equal(f(X, torch.zeros(n, n)), torch.zeros(n, n))
+    E = torch.zeros(n, n)
+    E[5, 141] = 1.0
+    R = f(E, X)
+    assert torch.equal(R[5], X[141]) and R.abs().sum() == X[141].abs().sum()
+    assert not torch.equal(f(X, X.T.contiguous()), f(X.T.contiguous(), X))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_accumulate_and_batch(hip, dtype):
+    b, M, N, K = 3, 256, 256, 128
+    A, B = _ints((b, M, K), 21, -1, 1, dtype), _ints((b, K, N), 22, -1, 1, dtype)
+    C0 = _ints((b, M, N), 23, -4, 4, torch.float32)
+    C = C0.clone().cuda()
+    hip.gemm(A.cuda(), B.cuda(), out=C, algo="strassen", accumulate=True)
+    assert torch.equal(C.cpu().double(), C0.double() + A.double() @ B.double())
+    C2 = hip.gemm(A.cuda(), B.cuda(), algo="winograd")
+    for i in range(b):  # batch independence
+        assert torch.equal(C2[i], hip.gemm(A[i].cuda(), B[i].cuda(), algo="winograd"))
+    # an edge-path shape with a broadcast B
+    A3 = _ints((b, 70, 50), 24, -1, 1, dtype)
+    B3 = _ints((50, 30), 25, -1, 1, dtype)
+    C3 = hip.gemm(A3.cuda(), B3.cuda().unsqueeze(0).expand(b, -1, -1), algo="strassen", out_dtype=torch.float32)
+    assert torch.equal(C3.cpu().double(), A3.double() @ B3.double())
+
+
+def test_config1_fp32_one_level_1024(hip):
+    """BASELINE config 1: 1024^3 fp32, N(0,1), one level."""
+    n = 1024
+    A, B = _gauss((n, n), 1234, 1.0, torch.float32), _gauss((n, n), 1235, 1.0, torch.float32)
+    import fixed_strassen
+    C = fixed_strassen._strassen_base(A.cuda(), B.cuda()).cpu()
+    ref = O.strassen_base(A, B)
+    assert O.rel_fro(C, ref) <= TOL[torch.float32]
+    assert O.rel_fro(C, A.double() @ B.double()) <= TOL[torch.float32]
+
+
+def test_config2_fp16_one_level_4096(hip):
+    """BASELINE config 2: 4096^3 fp16, N(0,1)/sqrt(K), fp32 aggregation, fp16 out."""
+    n = 4096
+    A = _gauss((n, n), 1234, n ** -0.5, torch.float16)
+    B = _gauss((n, n), 1235, n ** -0.5, torch.float16)
+    import fixed_strassen_fp32_agg as agg
+    C = agg._strassen_base(A.cuda(), B.cuda(), torch.float16).cpu()
+    assert C.dtype == torch.float16
+    ref = O.strassen_base_fp32_agg(A, B, torch.float16)
+    exact = A.double() @ B.double()
+    e_ref, e_exact = O.rel_fro(C, ref), O.rel_fro(C, exact)
+    print(f"config2: rel_fro vs oracle {e_ref:.3e}, vs fp64 {e_exact:.3e}, oracle vs fp64 {O.rel_fro(ref, exact):.3e}")
+    assert e_ref <= TOL[torch.float16] and e_exact <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("n_depth", [1, 2])
+def test_config3_bf16_8192(hip, n_depth):
+    """BASELINE config 3: 8192^3 bf16, N(0,1)/sqrt(K); two levels (49 products) and one level."""
+    n = 8192
+    A = _gauss((n, n), 1234, n ** -0.5, torch.bfloat16)
+    B = _gauss((n, n), 1235, n ** -0.5, torch.bfloat16)
+    import fixed_strassen_fp32_agg as agg
+    Ag, Bg = A.cuda(), B.cuda()
+    C = agg.strassen_matmul_n_layers(Ag, Bg, n_depth, torch.bfloat16)
+    assert C.dtype == torch.bfloat16
+    torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+    ref = O.strassen_matmul_n_layers(A, B, n_depth, torch.bfloat16, fp32_agg=True)
+    e_ref = O.rel_fro(C.cpu(), ref)
+    exact = torch.matmul(Ag.double(), Bg.double())   # fp64 classical product, on the GPU for speed
+    e_exact = float(torch.linalg.norm(C.double() - exact) / torch.linalg.norm(exact))
+    print(f"config3 depth {n_depth}: rel_fro vs oracle {e_ref:.3e}, vs fp64 {e_exact:.3e}")
+    assert e_ref <= TOL[torch.bfloat16] and e_exact <= TOL[torch.bfloat16]
+    # size-independent properties at full size: transposition and exact power-of-two scaling
+    Ct = agg.strassen_matmul_n_layers(Bg.T.contiguous(), Ag.T.contiguous(), n_depth, torch.bfloat16)
+    assert O.rel_fro(Ct.T.cpu(), C.cpu()) <= TOL[torch.bfloat16]
+    C4 = agg.strassen_matmul_n_layers(Ag * 4, Bg, n_depth, torch.bfloat16)
+    assert torch.equal(C4, C * 4)
+    assert torch.equal(C, agg.strassen_matmul_n_layers(Ag, Bg, n_depth, torch.bfloat16))  # run-to-run
+
+
+def test_config4_winograd_batched_bf16(hip):
+    """BASELINE config 4: batch 8 of 4096 x 8192 x 4096 bf16, U[-1,1]/sqrt(K), Winograd."""
+    b, M, K, N = 8, 4096, 8192, 4096
+    g = torch.Generator().manual_seed(1234)
+    A = ((torch.rand((b, M, K), generator=g) * 2 - 1) * K ** -0.5).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(1235)
+    B = ((torch.rand((b, K, N), generator=g) * 2 - 1) * K ** -0.5).to(torch.bfloat16)
+    Ag, Bg = A.cuda(), B.cuda()
+    C = hip.gemm(Ag, Bg, algo="winograd", levels=1)
+    assert C.shape == (b, M, N) and C.dtype == torch.bfloat16
+    torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+    for i in (0, 7):   # the oracle on two of the eight problems
+        ref = O.winograd_base(A[i], B[i], torch.bfloat16, fp32_agg=True)
+        assert O.rel_fro(C[i].cpu(), ref) <= TOL[torch.bfloat16]
+    exact = torch.matmul(Ag[3].double(), Bg[3].double())
+    assert float(torch.linalg.norm(C[3].double() - exact) / torch.linalg.norm(exact)) <= TOL[torch.bfloat16]
+    for i in range(b):  # batch independence at full size
+        assert torch.equal(C[i], hip.gemm(Ag[i], Bg[i], algo="winograd", levels=1))
+
+
+@pytest.mark.parametrize("d_in,d_out", [(768, 2304), (768, 768), (768, 3072), (3072, 768), (768, 769)])
+def test_config5_gpt2_linears(hip, d_in, d_out):
+    """BASELINE config 5: 8192 tokens, bf16 ~ N(0, 0.02): forward X W^T (NT), dgrad dY W (NN),
+    wgrad dY^T X (TN); 769 exercises the zero-padded odd size."""
+    T = 8192
+    X = _gauss((T, d_in), 1234, 0.02, torch.bfloat16)
+    W = _gauss((d_out, d_in), 1235, 0.02, torch.bfloat16)
+    dY = _gauss((T, d_out), 1236, 0.02, torch.bfloat16)
+    Xg, Wg, dYg = X.cuda(), W.cuda(), dY.cuda()
+    cases = {
+        "fwd": (Xg, Wg.T, X, W.T),
+        "dgrad": (dYg, Wg, dY, W),
+        "wgrad": (dYg.T, Xg, dY.T, X),
+    }
+    torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+    for name, (a, b, a_cpu, b_cpu) in cases.items():
+        C = hip.gemm(a, b, algo="strassen", levels=1)
+        ref = O.strassen_general(a_cpu.contiguous(), b_cpu.contiguous(), 1, torch.bfloat16, True)
+        exact = torch.matmul(a.double(), b.double())
+        e_ref = O.rel_fro(C.cpu(), ref)
+        e_exact = float(torch.linalg.norm(C.double() - exact) / torch.linalg.norm(exact))
+        assert e_ref <= TOL[torch.bfloat16] and e_exact <= TOL[torch.bfloat16], (name, e_ref, e_exact)
+
+
+def test_autograd_matmul(hip):
+    A = _ints((256, 128), 31, -1, 1).cuda().requires_grad_()
+    B = _ints((128, 384), 32, -1, 1).cuda().requires_grad_()
+    G = _ints((256, 384), 33, -1, 1).cuda()
+    hip.matmul(A, B).backward(G)
+    assert torch.equal(A.grad, G @ B.detach().T) and torch.equal(B.grad, A.detach().T @ G)

@@ -1,0 +1,91 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares,
+argument errors are reported without touching a GPU, and the host logic that mirrors the
+reference (recursion depth, validation, refusal of CPU tensors) behaves."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "strassen_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sthip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from strassen_hip import _capi
+    lib = _capi.load()
+    names = _header_symbols()
+    assert len(names) >= 8
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/strassen_hip.h but not exported"
+        assert n in _capi.SIGNATURES, f"{n} has no ctypes prototype"
+    assert set(_capi.SIGNATURES) == set(names)
+    assert lib.sthip_version() == 100
+
+
+def test_argument_errors_need_no_gpu():
+    from strassen_hip import _capi
+    lib = _capi.load()
+    s3 = (ctypes.c_int64 * 3)(0, 4, 1)
+    one = ctypes.c_void_p(16)
+    assert lib.sthip_gemm(one, one, one, 1, -1, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == -1
+    assert b"negative" in lib.sthip_last_error()
+    assert lib.sthip_gemm(one, one, one, 1, 4, 4, 4, s3, s3, s3, 7, 0, 1, 1, 0, None, 0, None) == -2
+    assert lib.sthip_gemm(one, one, one, 1, 4, 4, 4, s3, s3, s3, 2, 1, 1, 1, 0, None, 0, None) == -2
+    assert lib.sthip_gemm(one, one, one, 1, 4, 4, 4, s3, s3, s3, 0, 0, 9, 1, 0, None, 0, None) == -5
+    assert lib.sthip_gemm(None, one, one, 1, 4, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == -5
+    assert lib.sthip_gemm(one, one, one, 0, 4, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == 0   # empty batch
+    assert lib.sthip_gemm(one, one, one, 1, 0, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == 0   # empty M
+    assert lib.sthip_linear_strassen_forward(one, one, None, one, 9, 8, 0, 1, None, 0, None) == -1
+    assert b"cannot be padded" in lib.sthip_last_error()
+    # workspace: nothing for one level, S + M buffers for two
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == 0
+    two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
+    assert two == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4
+    three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
+    assert three == two + 2 * 256 * 256 * 2 + 7 * 256 * 256 * 4
+
+
+def test_reference_recursion_depth():
+    from _levels import practical_levels, reference_levels
+    # fixed_strassen.py:71-114 traced by hand
+    assert reference_levels(8192, 1) == 1 and reference_levels(8192, 2) == 2 and reference_levels(8192, 3) == 3
+    assert reference_levels(16, 1) == 0          # n <= 16 -> classical (:20-21)
+    assert reference_levels(32, 2) == 1          # halves of 16 are multiplied classically
+    assert reference_levels(64, 7) == 5          # the D=64, depth=7 demo (:173-184) stops at mid == 2
+    assert practical_levels(64, 5) == 1 and practical_levels(8192, 3) == 3 and practical_levels(32, 1) == 0
+
+
+def test_cpu_tensors_and_bad_shapes_are_refused():
+    import fixed_strassen
+    import fixed_strassen_fp32_agg
+    import strassen
+    import strassen_2_layer  # noqa: F401
+    from model.layers import LinearStrassen, replace_linear_with_strassen  # noqa: F401
+    assert fixed_strassen_fp32_agg.agg_dtype == torch.float32
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        fixed_strassen._strassen_base(torch.zeros(32, 32), torch.zeros(32, 32))
+    with pytest.raises(ValueError, match="square"):
+        strassen.strassen_matmul_two_layers(torch.zeros(8, 4), torch.zeros(4, 8))
+    with pytest.raises(ValueError, match="divisible by 4"):
+        strassen.strassen_matmul_two_layers(torch.zeros(6, 6), torch.zeros(6, 6))
+    with pytest.raises(AssertionError, match="square and a power of 2"):
+        LinearStrassen(96, 96, device="cpu")
+    lin = LinearStrassen(64, 64, device="cpu")
+    with pytest.raises(ValueError, match="Cannot pad input"):
+        lin(torch.zeros(65, 64))
+
+
+def test_product_code_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "strassen-triton_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)
