@@ -41,14 +41,184 @@ static const LaunchTable* table_for(int dt, int algo) {
     return nullptr;
 }
 
+static const LaunchTable2* table2_for(int dt, int algo) {
+    switch (dt * 3 + algo) {
+        case 3: return &kLaunch2_1_0; case 4: return &kLaunch2_1_1; case 5: return &kLaunch2_1_2;
+        case 6: return &kLaunch2_2_0; case 7: return &kLaunch2_2_1; case 8: return &kLaunch2_2_2;
+    }
+    return nullptr;
+}
+
+static int check_launch(const char* what);
+
 static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// ------------------------------------------------------------------ quadrant-sum pre-pass
+// out[o] = sum_q coef[o][q] * quadrant q, for up to five outputs at once, on matrices seen
+// in storage order (rows x cols, cols contiguous).  Each thread handles one 16-byte chunk
+// position: the four quadrant chunks are read once, every output is formed in fp32 and
+// rounded once to the operand type.
+struct ComboParams {
+    const void* q[4];
+    void* out[5];
+    int64_t ld_in, bs_in, ld_out, bs_out;   // elements
+    int nout, rows, chunks_per_row;
+    signed char coef[5][4];
+};
+
+template <class T>
+__global__ void quad_combos_kernel(const ComboParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
+    const int r = (int)(idx / p.chunks_per_row), c = (int)(idx % p.chunks_per_row);
+    const int64_t in_off = ((int64_t)blockIdx.y * p.bs_in + (int64_t)r * p.ld_in + c * 8) * 2;
+    const int64_t out_off = ((int64_t)blockIdx.y * p.bs_out + (int64_t)r * p.ld_out + c * 8) * 2;
+    u32x4 v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.q[q]) + in_off);
+    float x[4][8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t word = v[q][w];
+            if constexpr (__is_same(T, bf16_t)) { x[q][2 * w] = bf16lo(word); x[q][2 * w + 1] = bf16hi(word); }
+            else { const f16x2 h = as_f16x2(word); x[q][2 * w] = (float)h[0]; x[q][2 * w + 1] = (float)h[1]; }
+        }
+    for (int o = 0; o < p.nout; ++o) {
+        float s[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float acc = 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int cf = p.coef[o][q];
+                if (cf > 0) acc += x[q][e]; else if (cf < 0) acc -= x[q][e];
+            }
+            s[e] = acc;
+        }
+        u32x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (__is_same(T, bf16_t)) w[i] = pack_bf16(s[2 * i], s[2 * i + 1]);
+            else w[i] = pack_f16(s[2 * i], s[2 * i + 1]);
+        }
+        *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.out[o]) + out_off) = w;
+    }
+}
+
+// Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
+// Strassen (fixed_strassen.py:88-97): A side S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.
+static const signed char kStrA[5][4] = {{1, 1, 0, 0}, {0, 0, 1, 1}, {1, 0, 0, 1}, {0, 1, 0, -1}, {-1, 0, 1, 0}};
+static const signed char kStrB[5][4] = {{0, 1, 0, -1}, {-1, 0, 1, 0}, {1, 0, 0, 1}, {0, 0, 1, 1}, {1, 1, 0, 0}};
+// Winograd: A side S1 S2 S3 S4; B side T1 T2 T3 -T4.
+static const signed char kWinA[4][4] = {{0, 0, 1, 1}, {-1, 0, 1, 1}, {1, 0, -1, 0}, {1, 1, -1, -1}};
+static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0, 1}, {-1, 1, 1, -1}};
+
+static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
+    return (size_t)batch * 5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2));
+}
+
+static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
+    return dt != STHIP_F32 && Mh > 0 && Nh > 0 && Kh > 0 && Mh % 128 == 0 && Nh % 128 == 0 && Kh % kBK2 == 0;
+}
+
+// The pipelined path: optional quadrant-sum pre-pass into `ws`, then one grouped-GEMM launch.
+// Returns 1 if the problem does not qualify (the caller then takes the fused kernel).
+static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch, int64_t a_bs, int64_t b_bs,
+                            int64_t c_bs, int64_t Mh, int64_t Nh, int64_t Kh, int dt, bool out_f32, int algo,
+                            bool accumulate, bool a_kc, bool b_kc, char* ws, size_t ws_bytes, hipStream_t stream) {
+    const bool split = algo != STHIP_CLASSIC;
+    if (split && (!ws || !aligned_to(ws, 256) || ws_bytes < prepass_bytes(batch, Mh, Nh, Kh))) return 1;
+    const int64_t a_ld = a_kc ? A.rs : A.cs, b_ld = b_kc ? B.cs : B.rs;
+    Gemm2Params p;
+    memset(&p, 0, sizeof(p));
+    p.C = C; p.c_rs = c_rs; p.c_bs = c_bs;
+    p.Mh = (int)Mh; p.Nh = (int)Nh; p.Kh = (int)Kh;
+    p.tiles_m = (int)(Mh / 128); p.tiles_n = (int)(Nh / 128);
+    p.out_f32 = out_f32 ? 1 : 0; p.accumulate = accumulate ? 1 : 0; p.group_m = 8;
+    // raw quadrants in place
+    const char* Aq[4]; const char* Bq[4];
+    for (int q = 0; q < 4; ++q) {
+        Aq[q] = A.p + ((int64_t)(q >> 1) * Mh * A.rs + (int64_t)(q & 1) * Kh * A.cs) * 2;
+        Bq[q] = B.p + ((int64_t)(q >> 1) * Kh * B.rs + (int64_t)(q & 1) * Nh * B.cs) * 2;
+    }
+    if (!split) {
+        p.seg[0] = {A.p, B.p, a_ld, b_ld, a_bs, b_bs};
+    } else {
+        const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2);
+        char* SA = ws;                                // [5][batch] blocks of Mh x Kh (storage order of A)
+        char* SB = ws + (size_t)batch * 5 * sa_b;
+        const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
+        const int nout = algo == STHIP_STRASSEN ? 5 : 4;
+        for (int side = 0; side < 2; ++side) {
+            ComboParams cp;
+            memset(&cp, 0, sizeof(cp));
+            const bool kc = side == 0 ? a_kc : b_kc;
+            const int64_t r_ext = side == 0 ? (a_kc ? Mh : Kh) : (b_kc ? Nh : Kh);
+            const int64_t c_ext = side == 0 ? (a_kc ? Kh : Mh) : (b_kc ? Kh : Nh);
+            (void)kc;
+            for (int q = 0; q < 4; ++q) cp.q[q] = side == 0 ? Aq[q] : Bq[q];
+            for (int o = 0; o < nout; ++o) {
+                cp.out[o] = (side == 0 ? SA + (size_t)o * batch * sa_b : SB + (size_t)o * batch * sb_b);
+                for (int q = 0; q < 4; ++q)
+                    cp.coef[o][q] = algo == STHIP_STRASSEN ? (side == 0 ? kStrA[o][q] : kStrB[o][q])
+                                                           : (side == 0 ? kWinA[o][q] : kWinB[o][q]);
+            }
+            cp.ld_in = side == 0 ? a_ld : b_ld;
+            cp.bs_in = side == 0 ? a_bs : b_bs;
+            cp.ld_out = side == 0 ? sa_ld : sb_ld;
+            cp.bs_out = (int64_t)((side == 0 ? sa_b : sb_b) / 2);
+            cp.nout = nout; cp.rows = (int)r_ext; cp.chunks_per_row = (int)(c_ext / 8);
+            const int64_t n = r_ext * (c_ext / 8);
+            dim3 grid((unsigned)ceil_div(n, 256), (unsigned)batch);
+            if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, stream, cp);
+            else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, stream, cp);
+            int rc = check_launch("quad_combos");
+            if (rc) return rc;
+        }
+        const int64_t sa_bs = (int64_t)(sa_b / 2), sb_bs = (int64_t)(sb_b / 2);
+        auto SAo = [&](int o) { return (const void*)(SA + (size_t)o * batch * sa_b); };
+        auto SBo = [&](int o) { return (const void*)(SB + (size_t)o * batch * sb_b); };
+        auto rawA = [&](int q) { return Seg2{Aq[q], nullptr, a_ld, 0, a_bs, 0}; };
+        auto set = [&](int i, const void* a, int64_t ald, int64_t abs_, const void* b, int64_t bld, int64_t bbs) {
+            p.seg[i] = {a, b, ald, bld, abs_, bbs};
+        };
+        (void)rawA;
+        if (algo == STHIP_STRASSEN) {
+            // kernel order M3 M6 M5 M7 M1 M2 M4; A sums S2 S3 S5 S7 S9 = outputs 0..4, B sums S1 S4 S6 S8 S10
+            set(0, Aq[0], a_ld, a_bs, SBo(0), sb_ld, sb_bs);      // M3 = A11 S1
+            set(1, SAo(4), sa_ld, sa_bs, SBo(4), sb_ld, sb_bs);   // M6 = S9 S10
+            set(2, SAo(0), sa_ld, sa_bs, Bq[3], b_ld, b_bs);      // M5 = S2 B22
+            set(3, SAo(3), sa_ld, sa_bs, SBo(3), sb_ld, sb_bs);   // M7 = S7 S8
+            set(4, SAo(2), sa_ld, sa_bs, SBo(2), sb_ld, sb_bs);   // M1 = S5 S6
+            set(5, SAo(1), sa_ld, sa_bs, Bq[0], b_ld, b_bs);      // M2 = S3 B11
+            set(6, Aq[3], a_ld, a_bs, SBo(1), sb_ld, sb_bs);      // M4 = A22 S4
+        } else {
+            // kernel order P1 P2 P6 P7 P5 P3 -P4; A outputs S1..S4 = 0..3, B outputs T1 T2 T3 -T4 = 0..3
+            set(0, Aq[0], a_ld, a_bs, Bq[0], b_ld, b_bs);         // P1 = A11 B11
+            set(1, Aq[1], a_ld, a_bs, Bq[2], b_ld, b_bs);         // P2 = A12 B21
+            set(2, SAo(1), sa_ld, sa_bs, SBo(1), sb_ld, sb_bs);   // P6 = S2 T2
+            set(3, SAo(2), sa_ld, sa_bs, SBo(2), sb_ld, sb_bs);   // P7 = S3 T3
+            set(4, SAo(0), sa_ld, sa_bs, SBo(0), sb_ld, sb_bs);   // P5 = S1 T1
+            set(5, SAo(3), sa_ld, sa_bs, Bq[3], b_ld, b_bs);      // P3 = S4 B22
+            set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
+        }
+    }
+    const LaunchTable2* t = table2_for(dt, algo);
+    if (!t) return 1;
+    hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return STHIP_OK;
+}
 
 // One fused launch: C (+)= A x B with zero or one Strassen / Winograd level.
 // (Mh, Nh, Kh) is the block size used for the split; pass 0 to derive it from the sizes.
 static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                         int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
                         int64_t M, int64_t N, int64_t K, int64_t Mh, int64_t Nh, int64_t Kh,
-                        int dt, bool out_f32, int algo, bool accumulate, hipStream_t stream) {
+                        int dt, bool out_f32, int algo, bool accumulate, char* ws, size_t ws_bytes,
+                        hipStream_t stream) {
     if (M == 0 || N == 0 || batch == 0) return STHIP_OK;
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535)
         return fail(STHIP_ERR_SHAPE, "size out of range (M=%lld N=%lld K=%lld batch=%lld)",
@@ -93,6 +263,11 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     const bool whole = !split || (M == 2 * Mh && N == 2 * Nh && K == 2 * Kh);
     const bool fast = whole && Mh % kBM == 0 && Nh % kBN == 0 && Kh % bk == 0 && Kh > 0 && p.a_vec && p.b_vec && p.c_vec;
 
+    if (fast && fast_shape(dt, Mh, Nh, Kh) && a_long % 8 == 0 && b_long % 8 == 0) {
+        int rc = launch_pipelined(A, B, C, c_rs, batch, a_bs, b_bs, c_bs, Mh, Nh, Kh, dt, out_f32, algo, accumulate,
+                                  a_kc, b_kc, ws, ws_bytes, stream);
+        if (rc <= 0) return rc;
+    }
     const LaunchTable* t = table_for(dt, algo);
     if (!t) return fail(STHIP_ERR_ARG, "bad dtype/algo (%d, %d)", dt, algo);
     hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0][fast ? 0 : 1](p, (int)batch, stream);
@@ -218,8 +393,9 @@ static const Term kATerms[7] = {{0, 3, +1}, {2, 3, +1}, {0, 0, 0}, {3, 0, 0}, {0
 static const Term kBTerms[7] = {{0, 3, +1}, {0, 0, 0}, {1, 3, -1}, {2, 0, -1}, {3, 0, 0}, {0, 1, +1}, {2, 3, +1}};
 
 static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels) {
-    if (levels <= 1) return 0;
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
+    if (levels <= 0) return 0;
+    if (levels == 1) return fast_shape(dt, mh, nh, kh) ? prepass_bytes(1, mh, nh, kh) : 0;
     const size_t es = elem_size(dt);
     return align256(mh * kh * es) + align256(kh * nh * es) + 7 * align256(mh * nh * 4) +
            workspace_for(mh, nh, kh, dt, levels - 1);
@@ -233,10 +409,12 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                     char* ws, size_t ws_bytes, hipStream_t stream) {
     const bool out_f32 = out_dt == STHIP_F32;
     if (algo == STHIP_CLASSIC || levels <= 0)
-        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, 0, 0, 0, dt, out_f32, STHIP_CLASSIC, accumulate, stream);
+        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, 0, 0, 0, dt, out_f32, STHIP_CLASSIC, accumulate,
+                            nullptr, 0, stream);
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
     if (levels == 1)
-        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, mh, nh, kh, dt, out_f32, algo, accumulate, stream);
+        return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, mh, nh, kh, dt, out_f32, algo, accumulate,
+                            ws, ws_bytes, stream);
 
     const size_t es = elem_size(dt);
     const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es), m_b = align256(mh * nh * 4);
@@ -313,7 +491,8 @@ int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, 
         View a = {reinterpret_cast<const char*>(A), sA[1], sA[2]};
         View b = {reinterpret_cast<const char*>(B), sB[1], sB[2]};
         return launch_fused(a, b, reinterpret_cast<char*>(C), sC[1], sC[2], batch, sA[0], sB[0], sC[0], M, N, K,
-                            Mp / 2, Np / 2, Kp / 2, in_dtype, out_dtype == STHIP_F32, algo, accumulate != 0, s);
+                            Mp / 2, Np / 2, Kp / 2, in_dtype, out_dtype == STHIP_F32, algo, accumulate != 0,
+                            reinterpret_cast<char*>(workspace), workspace_bytes, s);
     }
     for (int64_t bi = 0; bi < batch; ++bi) {
         View a = {reinterpret_cast<const char*>(A) + bi * sA[0] * es, sA[1], sA[2]};
@@ -327,10 +506,14 @@ int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, 
 }
 
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {
-    (void)batch; (void)out_dtype;
-    if (algo == STHIP_CLASSIC || levels <= 1 || M <= 0 || N <= 0 || K < 0 || levels > 8 || in_dtype < 0 || in_dtype > 2) return 0;
+    (void)out_dtype;
+    if (algo == STHIP_CLASSIC || levels <= 0 || M <= 0 || N <= 0 || K < 0 || levels > 8 || in_dtype < 0 || in_dtype > 2) return 0;
     const int64_t q = (int64_t)1 << levels;
-    return workspace_for(round_up(M, q), round_up(N, q), round_up(K, q), in_dtype, levels);
+    const int64_t Mp = round_up(M, q), Np = round_up(N, q), Kp = round_up(K, q);
+    // one level: the batch goes into a single launch, so the pre-pass buffers scale with it (and
+    // only whole, tile-aligned problems take that path); deeper: batches run one after another
+    if (levels == 1) return (Mp == M && Np == N && Kp == K) ? (size_t)batch * workspace_for(Mp, Np, Kp, in_dtype, 1) : 0;
+    return workspace_for(Mp, Np, Kp, in_dtype, levels);
 }
 
 int sthip_strassen_matmul_n_layers(const void* A, const void* B, void* C, int64_t n,

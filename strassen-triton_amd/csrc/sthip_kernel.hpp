@@ -76,6 +76,9 @@ struct TileGeom {
 // ------------------------------------------------------------------ element arithmetic
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+// Taking the argument by value matters: __builtin_bit_cast applied directly to a vector
+// element expression reads element 0 whatever the index is.
+__device__ __forceinline__ f16x2 as_f16x2(uint32_t w) { return __builtin_bit_cast(f16x2, w); }
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     f32x2 f = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
@@ -106,9 +109,10 @@ __device__ __forceinline__ u32x4 combine(const u32x4 (&v)[NT]) {
         u32x4 r;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            f16x2 a = __builtin_bit_cast(f16x2, v[0][w]);
-            f16x2 b = __builtin_bit_cast(f16x2, v[1][w]);
-            r[w] = __builtin_bit_cast(uint32_t, (NEG & 2u) ? a - b : a + b);
+            const f16x2 a = as_f16x2(v[0][w]), b = as_f16x2(v[1][w]);
+            f16x2 c;
+            if constexpr ((NEG & 2u) != 0) c = a - b; else c = a + b;
+            r[w] = __builtin_bit_cast(uint32_t, c);
         }
         return r;
     } else {
@@ -123,7 +127,7 @@ __device__ __forceinline__ u32x4 combine(const u32x4 (&v)[NT]) {
                     xl = bf16lo(v[t][w]);
                     xh = bf16hi(v[t][w]);
                 } else {
-                    f16x2 h = __builtin_bit_cast(f16x2, v[t][w]);
+                    const f16x2 h = as_f16x2(v[t][w]);
                     xl = (float)h[0];
                     xh = (float)h[1];
                 }
@@ -426,7 +430,7 @@ __device__ __forceinline__ void store_tile(const Acc& acc, const GemmParams& P, 
                                 v[0] += bf16lo(old[0]); v[1] += bf16hi(old[0]);
                                 v[2] += bf16lo(old[1]); v[3] += bf16hi(old[1]);
                             } else if constexpr (__is_same(T, f16_t)) {
-                                f16x2 h0 = __builtin_bit_cast(f16x2, old[0]), h1 = __builtin_bit_cast(f16x2, old[1]);
+                                const f16x2 h0 = as_f16x2(old[0]), h1 = as_f16x2(old[1]);
                                 v[0] += (float)h0[0]; v[1] += (float)h0[1];
                                 v[2] += (float)h1[0]; v[3] += (float)h1[1];
                             }

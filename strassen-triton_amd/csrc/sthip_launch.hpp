@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "sthip_kernel.hpp"
+#include "sthip_kernel2.hpp"
 
 namespace sthip {
 
@@ -33,6 +34,31 @@ hipError_t launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads), C::SMEM_BYTES, stream, p);
+    return hipGetLastError();
+}
+
+// Pipelined kernel (16-bit operands): one table per (type, algorithm), indexed [a_kc][b_kc].
+typedef hipError_t (*LaunchFn2)(const Gemm2Params&, int batch, hipStream_t);
+struct LaunchTable2 { LaunchFn2 fn[2][2]; };
+#define STHIP_DECLARE_TABLE2(T, A) extern const LaunchTable2 kLaunch2_##T##_##A;
+STHIP_DECLARE_TABLE2(1, 0) STHIP_DECLARE_TABLE2(1, 1) STHIP_DECLARE_TABLE2(1, 2)
+STHIP_DECLARE_TABLE2(2, 0) STHIP_DECLARE_TABLE2(2, 1) STHIP_DECLARE_TABLE2(2, 2)
+#undef STHIP_DECLARE_TABLE2
+
+template <class T, int ALGO, bool A_KC, bool B_KC>
+hipError_t launch_gemm2(const Gemm2Params& p, int batch, hipStream_t stream) {
+    auto kern = gemm2_kernel<T, ALGO, A_KC, B_KC>;
+    static bool opted[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && !opted[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes2);
+        if (e != hipSuccess) return e;
+        opted[dev] = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads), kSmemBytes2, stream, p);
     return hipGetLastError();
 }
 

@@ -44,12 +44,19 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_gemm(one, one, one, 1, 0, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == 0   # empty M
     assert lib.sthip_linear_strassen_forward(one, one, None, one, 9, 8, 0, 1, None, 0, None) == -1
     assert b"cannot be padded" in lib.sthip_last_error()
-    # workspace: nothing for one level, S + M buffers for two
-    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == 0
+    # workspace.  One level: room for the ten quadrant sums (5 per operand) when the shape is
+    # tile aligned, per batch entry; nothing for fp32, odd or unaligned shapes, or classic.
+    sums = lambda h: 2 * 5 * h * h * 2
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == sums(512)
+    assert lib.sthip_workspace_bytes(3, 1024, 1024, 1024, 1, 1, 2, 1) == 3 * sums(512)
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == 0
+    assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
+    # Two levels: one S_A, one S_B and seven fp32 M buffers of half size, plus the leaf's sums.
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
-    assert two == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4
+    assert two == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4 + sums(256)
     three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
-    assert three == two + 2 * 256 * 256 * 2 + 7 * 256 * 256 * 4
+    assert three == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4 + 2 * 256 * 256 * 2 + 7 * 256 * 256 * 4 + sums(128)
 
 
 def test_reference_recursion_depth():
