@@ -34,6 +34,7 @@ WORKLOADS = {
     "strassen1_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "strassen", 1),
     "strassen2_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "strassen", 2),
     "classic_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "classic", 0),
+    "winograd1_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "winograd", 1),
     "strassen1_4096_f16": (1, 4096, 4096, 4096, torch.float16, "strassen", 1),
     "strassen1_1024_f32": (1, 1024, 1024, 1024, torch.float32, "strassen", 1),
     "winograd_b8_4096x8192x4096_bf16": (8, 4096, 4096, 8192, torch.bfloat16, "winograd", 1),

@@ -38,6 +38,10 @@ def _units():
         for a in range(3):
             units.append((f"sthip_inst2_{t}_{a}.o", "sthip_inst2.hip",
                           [f"-DSTHIP_INST_TYPE={t}", f"-DSTHIP_INST_ALGO={a}"]))
+    for t in (1, 2):
+        for a in range(3):
+            units.append((f"sthip_inst3_{t}_{a}.o", "sthip_inst3.hip",
+                          [f"-DSTHIP_INST_TYPE={t}", f"-DSTHIP_INST_ALGO={a}"]))
     return units
 
 

@@ -51,6 +51,14 @@ static const LaunchTable2* table2_for(int dt, int algo) {
 
 static int check_launch(const char* what);
 
+static const LaunchTable3* table3_for(int dt, int algo) {
+    switch (dt * 3 + algo) {
+        case 3: return &kLaunch3_1_0; case 4: return &kLaunch3_1_1; case 5: return &kLaunch3_1_2;
+        case 6: return &kLaunch3_2_0; case 7: return &kLaunch3_2_1; case 8: return &kLaunch3_2_2;
+    }
+    return nullptr;
+}
+
 static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // ------------------------------------------------------------------ quadrant-sum pre-pass
@@ -115,8 +123,10 @@ static const signed char kStrB[5][4] = {{0, 1, 0, -1}, {-1, 0, 1, 0}, {1, 0, 0, 
 static const signed char kWinA[4][4] = {{0, 0, 1, 1}, {-1, 0, 1, 1}, {1, 0, -1, 0}, {1, 1, -1, -1}};
 static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0, 1}, {-1, 1, 1, -1}};
 
+// Workspace of the pipelined path per problem: five sums per operand plus one fp32 tile per
+// workgroup for the accumulator the 256 x 128 Strassen kernel parks (Mh x Nh floats in all).
 static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
-    return (size_t)batch * 5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2));
+    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + align256(Mh * Nh * 4));
 }
 
 static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
@@ -149,6 +159,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2);
         char* SA = ws;                                // [5][batch] blocks of Mh x Kh (storage order of A)
         char* SB = ws + (size_t)batch * 5 * sa_b;
+        p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
         const int nout = algo == STHIP_STRASSEN ? 5 : 4;
         for (int side = 0; side < 2; ++side) {
@@ -205,9 +216,19 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
         }
     }
-    const LaunchTable2* t = table2_for(dt, algo);
-    if (!t) return 1;
-    hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+    // Fixed tile table: 256 x 128 tiles (less global->LDS traffic per flop) whenever A is
+    // contiguous along k and the block height allows it, 128 x 128 tiles otherwise.
+    hipError_t e;
+    const LaunchTable3* t3 = table3_for(dt, algo);
+    if (a_kc && Mh % kBM3 == 0 && t3) {
+        p.tiles_m = (int)(Mh / kBM3);
+        p.group_m = 4;
+        e = t3->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+    } else {
+        const LaunchTable2* t = table2_for(dt, algo);
+        if (!t) return 1;
+        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+    }
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
     return STHIP_OK;
 }
