@@ -81,12 +81,21 @@ def cpu_baseline(A, B, levels, dtype, algo):
         A, B = A[0], B[0]
     M, K = A.shape
     N = B.shape[1]
+    # torch's CPU GEMM for bf16/fp16 is fast only with AMX / AVX512-FP16; probe it and fall back
+    # to the same recursion with fp32-upcast leaf products (sgemm) where it is not
+    leaf, leaf_name = torch.mm, "native " + DT_NAME[dtype] + " leaf products"
+    if dtype != torch.float32:
+        P = torch.ones(1024, 1024, dtype=dtype)
+        t0 = time.perf_counter()
+        torch.mm(P, P)
+        if time.perf_counter() - t0 > 0.25:     # < ~8 GFLOP/s
+            leaf, leaf_name = O.mm_fp32_upcast, "fp32-upcast leaf products (native 16-bit CPU GEMM too slow here)"
     if algo == "winograd":
-        f = lambda: O.winograd_base(A, B, dtype, fp32_agg=True)
+        f = lambda: O.winograd_base(A, B, dtype, fp32_agg=True, mm=leaf)
     elif algo == "classic":
-        f = lambda: torch.matmul(A, B)
+        f = lambda: leaf(A, B)
     else:
-        f = lambda: O.strassen_matmul_n_layers(A, B, levels, dtype, fp32_agg=True)
+        f = lambda: O.strassen_matmul_n_layers(A, B, levels, dtype, fp32_agg=True, mm=leaf)
     f()
     best = float("inf")
     spent = 0.0
@@ -99,7 +108,7 @@ def cpu_baseline(A, B, levels, dtype, algo):
             break
     return {"value": round(2.0 * M * N * K / best / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"one {M}x{N}x{K} {DT_NAME[dtype]} product through the CPU oracle "
-                      f"({algo}, {levels} level(s), fp32 aggregation), best of 3 after 1 warm-up; "
+                      f"({algo}, {levels} level(s), fp32 aggregation, {leaf_name}), best of 3 after 1 warm-up; "
                       f"best {best * 1e3:.1f} ms"}
 
 

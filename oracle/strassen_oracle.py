@@ -21,15 +21,24 @@ matrix-level Strassen recursion.  Every function names the reference lines it fo
                                (strassen_deprecated_winograd.py:461-472 only gets C11 right),
                                so this one is pinned by the identity C = A @ B alone.
 
-Pinning.  The reference ships no golden vectors or tests.  What fixes these functions
-is mathematics: in exact arithmetic each of them equals A @ B, so the tests run them on
-small-integer matrices (every partial sum exactly representable) and demand bit-equality
-with an fp64 classical product; on tiny sizes against a triple loop; on identity, zero,
-one-hot and block-diagonal inputs; and through transposition / linearity invariants.  A
-dropped term, wrong sign, swapped quadrant or transposed operand fails at least one of
-those.  What mathematics cannot fix is *where* the reference rounds to bf16/fp16 (the
-cast schedule of fixed_strassen_fp32_agg.py); that part is read off the source text
-and is "parity unpinned" at the bit level -- comparisons against it are tolerance based
+Pinning.  The reference ships no golden vectors or tests of its own, so the oracle is
+pinned twice over:
+  * formulas -- in exact arithmetic every function here equals A @ B, so tests/test_oracle.py
+    runs them on small-integer matrices (every partial sum exactly representable) and
+    demands bit-equality with an fp64 classical product; on tiny sizes against a triple
+    loop; on identity, zero, one-hot and block-diagonal inputs; and through transposition /
+    linearity invariants.  A dropped term, wrong sign, swapped quadrant or transposed
+    operand fails at least one of those.
+  * cast schedule (where the reference rounds to bf16 / fp16 / fp32) -- mathematics cannot
+    fix that, so tests/golden/reference_cast_schedule.npz holds outputs of the reference's own
+    fixed_strassen.py / fixed_strassen_fp32_agg.py functions (run eagerly on CPU by
+    tests/golden/make_reference_vectors.py) and tests/test_golden_reference.py demands that
+    strassen_base, strassen_base_fp32_agg and strassen_matmul_n_layers reproduce them bit
+    for bit (fp32, bf16, fp16; depth 1-3; n = 32, 64, 128).
+Not covered by reference vectors, because the reference has no counterpart: winograd_base and
+strassen_general (rectangular / batched / odd sizes).  Their formulas are pinned by the
+identity tests above; their cast schedule is this file's own choice (the fp32_agg schedule
+applied to the new shapes) -- "parity unpinned" at the bit level, compared by tolerance
 (rel. Frobenius <= 1e-5 fp32, <= 2e-2 bf16/fp16).
 """
 from __future__ import annotations
@@ -43,6 +52,17 @@ AGG_DTYPE = torch.float32  # fixed_strassen_fp32_agg.py:10
 LEAF = 16
 
 
+def mm_fp32_upcast(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """x @ y for 16-bit operands computed as an fp32 product of the upcast operands, rounded
+    once to the operand dtype.  Same arithmetic contract as a half-precision GEMM with fp32
+    accumulation, but it runs through sgemm: torch's CPU fp16 matmul is hundreds of times
+    slower, which matters for the 4096 / 8192 test sizes.  Not bit-identical to torch.mm on
+    16-bit tensors (summation order differs); use it for tolerance comparisons only."""
+    if x.dtype == torch.float32 and y.dtype == torch.float32:
+        return torch.matmul(x, y)
+    return torch.matmul(x.float(), y.float()).to(x.dtype)
+
+
 def _quadrants(X: torch.Tensor, mid_r: int, mid_c: int):
     return (X[..., :mid_r, :mid_c], X[..., :mid_r, mid_c:],
             X[..., mid_r:, :mid_c], X[..., mid_r:, mid_c:])
@@ -53,7 +73,7 @@ def _assemble(C11, C12, C21, C22):
     return torch.cat([torch.cat([C11, C12], dim=-1), torch.cat([C21, C22], dim=-1)], dim=-2)
 
 
-def strassen_base(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+def strassen_base(A: torch.Tensor, B: torch.Tensor, mm=torch.mm) -> torch.Tensor:
     """One Strassen level, every add and product in the dtype of the inputs.
 
     Follows fixed_strassen.py:11-57: n = A.shape[0]; n <= 16 -> plain product (:20-21);
@@ -61,17 +81,17 @@ def strassen_base(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
     C11 = M1+M4-M5+M7, C12 = M3+M5, C21 = M2+M4, C22 = M1-M2+M3+M6 (:48-51).
     """
     if A.shape[0] <= LEAF:
-        return torch.mm(A, B)
+        return mm(A, B)
     mid = A.shape[0] // 2
     A11, A12, A21, A22 = _quadrants(A, mid, mid)
     B11, B12, B21, B22 = _quadrants(B, mid, mid)
-    M1 = torch.mm(A11 + A22, B11 + B22)
-    M2 = torch.mm(A21 + A22, B11)
-    M3 = torch.mm(A11, B12 - B22)
-    M4 = torch.mm(A22, B21 - B11)
-    M5 = torch.mm(A11 + A12, B22)
-    M6 = torch.mm(A21 - A11, B11 + B12)
-    M7 = torch.mm(A12 - A22, B21 + B22)
+    M1 = mm(A11 + A22, B11 + B22)
+    M2 = mm(A21 + A22, B11)
+    M3 = mm(A11, B12 - B22)
+    M4 = mm(A22, B21 - B11)
+    M5 = mm(A11 + A12, B22)
+    M6 = mm(A21 - A11, B11 + B12)
+    M7 = mm(A12 - A22, B21 + B22)
     C11 = M1 + M4 - M5 + M7
     C12 = M3 + M5
     C21 = M2 + M4
@@ -80,7 +100,7 @@ def strassen_base(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
 
 
 def strassen_base_fp32_agg(A: torch.Tensor, B: torch.Tensor,
-                           base_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                           base_dtype: torch.dtype = torch.float32, mm=torch.mm) -> torch.Tensor:
     """One Strassen level with fp32 sums and fp32 recombination.
 
     Follows fixed_strassen_fp32_agg.py:12-56: quadrants upcast to fp32 (:26-35); each
@@ -88,21 +108,21 @@ def strassen_base_fp32_agg(A: torch.Tensor, B: torch.Tensor,
     base_dtype) upcast again (:38-44); recombination in fp32, one final rounding (:47-50).
     """
     if A.shape[0] <= LEAF:
-        return torch.mm(A, B)
+        return mm(A, B)
     mid = A.shape[0] // 2
     A11, A12, A21, A22 = (q.to(AGG_DTYPE) for q in _quadrants(A, mid, mid))
     B11, B12, B21, B22 = (q.to(AGG_DTYPE) for q in _quadrants(B, mid, mid))
 
-    def mm(x, y):
-        return torch.mm(x.to(base_dtype), y.to(base_dtype)).to(AGG_DTYPE)
+    def prod(x, y):
+        return mm(x.to(base_dtype), y.to(base_dtype)).to(AGG_DTYPE)
 
-    M1 = mm(A11 + A22, B11 + B22)
-    M2 = mm(A21 + A22, B11)
-    M3 = mm(A11, B12 - B22)
-    M4 = mm(A22, B21 - B11)
-    M5 = mm(A11 + A12, B22)
-    M6 = mm(A21 - A11, B11 + B12)
-    M7 = mm(A12 - A22, B21 + B22)
+    M1 = prod(A11 + A22, B11 + B22)
+    M2 = prod(A21 + A22, B11)
+    M3 = prod(A11, B12 - B22)
+    M4 = prod(A22, B21 - B11)
+    M5 = prod(A11 + A12, B22)
+    M6 = prod(A21 - A11, B11 + B12)
+    M7 = prod(A12 - A22, B21 + B22)
     C11 = (M1 + M4 - M5 + M7).to(base_dtype)
     C12 = (M3 + M5).to(base_dtype)
     C21 = (M2 + M4).to(base_dtype)
@@ -113,7 +133,7 @@ def strassen_base_fp32_agg(A: torch.Tensor, B: torch.Tensor,
 def strassen_matmul_n_layers(A: torch.Tensor, B: torch.Tensor, n_depth: int = 2,
                              base_dtype: torch.dtype = torch.float32, *,
                              fp32_agg: bool = False,
-                             inner_keeps_base_dtype: bool = False) -> torch.Tensor:
+                             inner_keeps_base_dtype: bool = False, mm=torch.mm) -> torch.Tensor:
     """n_depth-level recursion.
 
     fp32_agg=False follows fixed_strassen.py:59-126 (base_dtype ignored, math in the
@@ -128,23 +148,24 @@ def strassen_matmul_n_layers(A: torch.Tensor, B: torch.Tensor, n_depth: int = 2,
     """
     if not fp32_agg:
         if n_depth == 1:
-            return strassen_base(A, B)
+            return strassen_base(A, B, mm)
         mid = A.shape[0] // 2
         A11, A12, A21, A22 = _quadrants(A, mid, mid)
         B11, B12, B21, B22 = _quadrants(B, mid, mid)
         S1, S2, S3, S4, S5 = B12 - B22, A11 + A12, A21 + A22, B21 - B11, A11 + A22
         S6, S7, S8, S9, S10 = B11 + B22, A12 - A22, B21 + B22, A21 - A11, B11 + B12
         if mid == 2 or n_depth == 2:
-            f = strassen_base
+            def f(x, y):
+                return strassen_base(x, y, mm)
         else:
             def f(x, y):
-                return strassen_matmul_n_layers(x, y, n_depth - 1)
+                return strassen_matmul_n_layers(x, y, n_depth - 1, mm=mm)
         M1, M2, M3, M4 = f(S5, S6), f(S3, B11), f(A11, S1), f(A22, S4)
         M5, M6, M7 = f(S2, B22), f(S9, S10), f(S7, S8)
         return _assemble(M1 + M4 - M5 + M7, M3 + M5, M2 + M4, M1 - M2 + M3 + M6)
 
     if n_depth == 1:
-        return strassen_base_fp32_agg(A, B, base_dtype)
+        return strassen_base_fp32_agg(A, B, base_dtype, mm)
     mid = A.shape[0] // 2
     A11, A12, A21, A22 = (q.to(AGG_DTYPE) for q in _quadrants(A, mid, mid))
     B11, B12, B21, B22 = (q.to(AGG_DTYPE) for q in _quadrants(B, mid, mid))
@@ -154,12 +175,12 @@ def strassen_matmul_n_layers(A: torch.Tensor, B: torch.Tensor, n_depth: int = 2,
     inner_dtype = base_dtype if inner_keeps_base_dtype else torch.float32
     if mid == 2 or n_depth == 2:
         def f(x, y):
-            return strassen_base_fp32_agg(x, y, inner_dtype).to(AGG_DTYPE)
+            return strassen_base_fp32_agg(x, y, inner_dtype, mm).to(AGG_DTYPE)
     else:
         def f(x, y):
             return strassen_matmul_n_layers(
                 x, y, n_depth - 1, inner_dtype, fp32_agg=True,
-                inner_keeps_base_dtype=inner_keeps_base_dtype).to(AGG_DTYPE)
+                inner_keeps_base_dtype=inner_keeps_base_dtype, mm=mm).to(AGG_DTYPE)
     M1, M2, M3, M4 = f(S5, S6), f(S3, r(B11)), f(r(A11), S1), f(r(A22), S4)
     M5, M6, M7 = f(S2, r(B22)), f(S9, S10), f(S7, S8)
     return _assemble(r(M1 + M4 - M5 + M7), r(M3 + M5), r(M2 + M4), r(M1 - M2 + M3 + M6))
@@ -235,7 +256,7 @@ def strassen2_zorder_49(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
 
 
 def winograd_base(A: torch.Tensor, B: torch.Tensor, base_dtype: torch.dtype | None = None,
-                  fp32_agg: bool = True) -> torch.Tensor:
+                  fp32_agg: bool = True, mm=torch.matmul) -> torch.Tensor:
     """One level of Strassen-Winograd (7 products, 15 additions), rectangular allowed
     (even dimensions), batched allowed.
 
@@ -262,11 +283,11 @@ def winograd_base(A: torch.Tensor, B: torch.Tensor, base_dtype: torch.dtype | No
     T3 = B22 - B12
     T4 = T2 - B21
 
-    def mm(x, y):
-        return up(torch.matmul(x.to(base_dtype), y.to(base_dtype)))
+    def prod(x, y):
+        return up(mm(x.to(base_dtype), y.to(base_dtype)))
 
-    P1, P2, P3, P4 = mm(A11, B11), mm(A12, B21), mm(S4, B22), mm(A22, T4)
-    P5, P6, P7 = mm(S1, T1), mm(S2, T2), mm(S3, T3)
+    P1, P2, P3, P4 = prod(A11, B11), prod(A12, B21), prod(S4, B22), prod(A22, T4)
+    P5, P6, P7 = prod(S1, T1), prod(S2, T2), prod(S3, T3)
     U2 = P1 + P6
     U3 = U2 + P7
     U4 = U2 + P5
@@ -286,10 +307,10 @@ def _pad_to(X: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
     return torch.nn.functional.pad(X, (0, pc, 0, pr))
 
 
-def _strassen_rect_level(A, B, levels, base_dtype, fp32_agg):
+def _strassen_rect_level(A, B, levels, base_dtype, fp32_agg, mm=torch.matmul):
     """One-or-more levels on (possibly batched) rectangular operands with even dims."""
     if levels == 0:
-        return torch.matmul(A.to(base_dtype), B.to(base_dtype))
+        return mm(A.to(base_dtype), B.to(base_dtype))
     M, K = A.shape[-2:]
     N = B.shape[-1]
     up = (lambda t: t.to(AGG_DTYPE)) if fp32_agg else (lambda t: t)
@@ -298,7 +319,7 @@ def _strassen_rect_level(A, B, levels, base_dtype, fp32_agg):
     B11, B12, B21, B22 = (up(q) for q in _quadrants(B, K // 2, N // 2))
 
     def f(x, y):
-        return up(_strassen_rect_level(rd(x), rd(y), levels - 1, base_dtype, fp32_agg))
+        return up(_strassen_rect_level(rd(x), rd(y), levels - 1, base_dtype, fp32_agg, mm))
 
     M1 = f(A11 + A22, B11 + B22)
     M2 = f(A21 + A22, B11)
@@ -312,7 +333,7 @@ def _strassen_rect_level(A, B, levels, base_dtype, fp32_agg):
 
 def strassen_general(A: torch.Tensor, B: torch.Tensor, levels: int = 1,
                      base_dtype: torch.dtype | None = None, fp32_agg: bool = True,
-                     winograd: bool = False) -> torch.Tensor:
+                     winograd: bool = False, mm=torch.matmul) -> torch.Tensor:
     """(batch,) M x K times (batch,) K x N with `levels` Strassen levels, any sizes.
 
     Same formulas and cast schedule as strassen_base[_fp32_agg] / winograd_base, applied
@@ -329,9 +350,9 @@ def strassen_general(A: torch.Tensor, B: torch.Tensor, levels: int = 1,
     Ap, Bp = _pad_to(A, Mp, Kp), _pad_to(B, Kp, Np)
     if winograd:
         assert levels == 1
-        C = winograd_base(Ap, Bp, base_dtype, fp32_agg)
+        C = winograd_base(Ap, Bp, base_dtype, fp32_agg, mm)
     else:
-        C = _strassen_rect_level(Ap, Bp, levels, base_dtype, fp32_agg)
+        C = _strassen_rect_level(Ap, Bp, levels, base_dtype, fp32_agg, mm)
     return C[..., :M, :N].contiguous()
 
 

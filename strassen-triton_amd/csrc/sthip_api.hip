@@ -216,11 +216,13 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
         }
     }
-    // Fixed tile table: 256 x 128 tiles (less global->LDS traffic per flop) whenever A is
-    // contiguous along k and the block height allows it, 128 x 128 tiles otherwise.
+    // Fixed tile table: 256 x 128 tiles (less global->LDS traffic per flop) when A is contiguous
+    // along k, the block height allows it and there is a tile for every one of the 256 CUs;
+    // 128 x 128 tiles otherwise.
     hipError_t e;
     const LaunchTable3* t3 = table3_for(dt, algo);
-    if (a_kc && Mh % kBM3 == 0 && t3) {
+    const int64_t big_tiles = (Mh / kBM3) * (Nh / kBN3) * batch;
+    if (a_kc && Mh % kBM3 == 0 && t3 && big_tiles >= 256) {   // at least one 256 x 128 tile per CU
         p.tiles_m = (int)(Mh / kBM3);
         p.group_m = 4;
         e = t3->fn[b_kc ? 1 : 0](p, (int)batch, stream);

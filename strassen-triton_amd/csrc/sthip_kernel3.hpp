@@ -148,10 +148,12 @@ struct Pipe3 {
 
     __device__ __forceinline__ void read_frags(int buf, int sl, int kg) {
         const char* s = smem + sl * kStageBytes3;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) fa[buf][i] = read_frag3<true>(s, wm + i * 32, kg);
+        // B first: both B fragments feed the first two MFMAs of the k-group, A fragment i only
+        // MFMAs 2i and 2i+1, so this order gives every read the longest head start.
 #pragma unroll
         for (int j = 0; j < 2; ++j) fb[buf][j] = read_frag3<B_KC>(s + kATile3, wn + j * 32, kg);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[buf][i] = read_frag3<true>(s, wm + i * 32, kg);
     }
 
     __device__ __forceinline__ void start() {
@@ -195,6 +197,17 @@ struct Pipe3 {
                         if (!(STHIP_DBG & 64)) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                         else acc.t[i][j][0] += __builtin_bit_cast(float, fa[cb][i][0] ^ fb[cb][j][0]);   // experiment
                     }
+                // Pin the software pipeline: the fragment reads of the next k-group are spread one
+                // per MFMA of this k-group, so their LDS latency hides behind matrix-core time
+                // instead of being sunk next to their first use.
+                if (!(STHIP_DBG & 128)) {
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             slot = next_slot(slot);
         }

@@ -144,8 +144,10 @@ def test_config2_fp16_one_level_4096(hip):
     import fixed_strassen_fp32_agg as agg
     C = agg._strassen_base(A.cuda(), B.cuda(), torch.float16).cpu()
     assert C.dtype == torch.float16
-    ref = O.strassen_base_fp32_agg(A, B, torch.float16)
-    exact = A.double() @ B.double()
+    # CPU oracle with its leaf products through sgemm (torch's CPU fp16 matmul is far too slow
+    # at this size); the fp64 classical product comes from the GPU
+    ref = O.strassen_base_fp32_agg(A, B, torch.float16, mm=O.mm_fp32_upcast)
+    exact = torch.matmul(A.cuda().double(), B.cuda().double()).cpu()
     e_ref, e_exact = O.rel_fro(C, ref), O.rel_fro(C, exact)
     print(f"config2: rel_fro vs oracle {e_ref:.3e}, vs fp64 {e_exact:.3e}, oracle vs fp64 {O.rel_fro(ref, exact):.3e}")
     assert e_ref <= TOL[torch.float16] and e_exact <= TOL[torch.float16]
@@ -162,7 +164,7 @@ def test_config3_bf16_8192(hip, n_depth):
     C = agg.strassen_matmul_n_layers(Ag, Bg, n_depth, torch.bfloat16)
     assert C.dtype == torch.bfloat16
     torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
-    ref = O.strassen_matmul_n_layers(A, B, n_depth, torch.bfloat16, fp32_agg=True)
+    ref = O.strassen_matmul_n_layers(A, B, n_depth, torch.bfloat16, fp32_agg=True, mm=O.mm_fp32_upcast)
     e_ref = O.rel_fro(C.cpu(), ref)
     exact = torch.matmul(Ag.double(), Bg.double())   # fp64 classical product, on the GPU for speed
     e_exact = float(torch.linalg.norm(C.double() - exact) / torch.linalg.norm(exact))
@@ -188,7 +190,7 @@ def test_config4_winograd_batched_bf16(hip):
     assert C.shape == (b, M, N) and C.dtype == torch.bfloat16
     torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
     for i in (0, 7):   # the oracle on two of the eight problems
-        ref = O.winograd_base(A[i], B[i], torch.bfloat16, fp32_agg=True)
+        ref = O.winograd_base(A[i], B[i], torch.bfloat16, fp32_agg=True, mm=O.mm_fp32_upcast)
         assert O.rel_fro(C[i].cpu(), ref) <= TOL[torch.bfloat16]
     exact = torch.matmul(Ag[3].double(), Bg[3].double())
     assert float(torch.linalg.norm(C[3].double() - exact) / torch.linalg.norm(exact)) <= TOL[torch.bfloat16]
@@ -213,7 +215,7 @@ def test_config5_gpt2_linears(hip, d_in, d_out):
     torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
     for name, (a, b, a_cpu, b_cpu) in cases.items():
         C = hip.gemm(a, b, algo="strassen", levels=1)
-        ref = O.strassen_general(a_cpu.contiguous(), b_cpu.contiguous(), 1, torch.bfloat16, True)
+        ref = O.strassen_general(a_cpu.contiguous(), b_cpu.contiguous(), 1, torch.bfloat16, True, mm=O.mm_fp32_upcast)
         exact = torch.matmul(a.double(), b.double())
         e_ref = O.rel_fro(C.cpu(), ref)
         e_exact = float(torch.linalg.norm(C.double() - exact) / torch.linalg.norm(exact))
