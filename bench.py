@@ -1,20 +1,30 @@
 """Benchmark of the Strassen hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
-A step is one C = A @ B through the fused one-level Strassen kernel (the C-ABI call, inputs
-resident in HBM).  The default workload is the one BASELINE.json's metric is quoted on:
+A step is one C = A @ B through the library's C ABI with the inputs resident in HBM.  The
+default workload is the one BASELINE.json's metric is quoted on: one-level Strassen,
 M = N = K = 8192, bf16 in / bf16 out, fp32 accumulation and aggregation.  Prints ONE JSON
-line: effective TFLOP/s (2MNK / t, the classical flop count, as the reference's
-main_profiling.py:190,216-217 does), the ratio to a hipBLASLt classical GEMM of the same
-shape timed the same way, the MFMA roofline fraction of the Strassen kernel, and the CPU
-oracle timed on the host cores.
+line:
+
+  value / ms_per_step   effective TFLOP/s = 2MNK / t (the classical flop count, as the
+                        reference's main_profiling.py:190,216-217 counts it) over exactly K
+                        back-to-back steps between two synchronisations
+  hipblaslt_*           torch.matmul (hipBLASLt) on the same tensors, same protocol, and the ratio
+  roofline              the dominant kernel (the grouped-GEMM launch) timed alone with HIP events
+                        on the stream it runs on, against the MI355X dense MFMA peak
+  cpu_baseline          the CPU oracle (a restatement of the reference's torch recursion) on the
+                        host cores, best of 3
+
+`--workload copy_1gib` runs a plain 1 GiB device copy instead; it exists to calibrate the
+FETCH_SIZE / WRITE_SIZE counters when the HBM traffic of the kernels is measured with rocprofv3.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -30,7 +40,7 @@ import torch  # noqa: E402
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA, vendor figures
 
 WORKLOADS = {
-    # name: (batch, M, N, K, dtype, algo, levels, input scale rule)
+    # name: (batch, M, N, K, dtype, algo, levels)
     "strassen1_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "strassen", 1),
     "strassen2_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "strassen", 2),
     "classic_8192_bf16": (1, 8192, 8192, 8192, torch.bfloat16, "classic", 0),
@@ -39,6 +49,7 @@ WORKLOADS = {
     "strassen1_1024_f32": (1, 1024, 1024, 1024, torch.float32, "strassen", 1),
     "winograd_b8_4096x8192x4096_bf16": (8, 4096, 4096, 8192, torch.bfloat16, "winograd", 1),
     "strassen1_16384_bf16": (1, 16384, 16384, 16384, torch.bfloat16, "strassen", 1),
+    "copy_1gib": None,
 }
 DT_NAME = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
 
@@ -55,8 +66,8 @@ def make_inputs(batch, M, N, K, dtype):
 
 
 def time_gpu(fn, steps, warmup):
-    """W untimed calls, then exactly K calls between two synchronisations; also HIP events on
-    the stream the kernels run on, for the per-launch duration."""
+    """W untimed calls, then exactly K calls between two synchronisations.  Returns the wall
+    time and the HIP-event time of the K calls (events recorded on the stream fn launches on)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -112,6 +123,28 @@ def cpu_baseline(A, B, levels, dtype, algo):
                       f"best {best * 1e3:.1f} ms"}
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE and recorded in profiles/ (None if no such summary is committed)."""
+    path = os.path.join(ROOT, "profiles", f"gemm_kernel_{workload}_hbm_traffic.txt")
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def copy_calibration(steps):
+    """A plain device copy of known size: 1 GiB read + 1 GiB written per step."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    wall, ev = time_gpu(lambda: dst.copy_(src), steps, 2)
+    print(json.dumps({"workload": "copy_1gib", "bytes_read_per_step": n, "bytes_written_per_step": n,
+                      "steps": steps, "ms_per_step": round(ev / steps * 1e3, 4),
+                      "GBps": round(2 * n * steps / ev / 1e9, 1)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -126,20 +159,37 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "copy_1gib":
+        copy_calibration(args.steps)
+        return
     import strassen_hip
     from strassen_hip import _capi
-    _capi.load()
+    lib = _capi.load()
 
     batch, M, N, K, dtype, algo, levels = WORKLOADS[args.workload]
     A, B = make_inputs(batch, M, N, K, dtype)
     Ag, Bg = A.cuda(), B.cuda()
     out = torch.empty(Ag.shape[:-1] + (N,), dtype=dtype, device="cuda")
     flops = 2.0 * batch * M * N * K
+    nbytes = strassen_hip.workspace_bytes(Ag, Bg, algo=algo, levels=levels)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device="cuda")
 
-    fn = lambda: strassen_hip.gemm(Ag, Bg, out=out, algo=algo, levels=levels)
+    fn = lambda: strassen_hip.gemm(Ag, Bg, out=out, algo=algo, levels=levels, workspace=ws)
     wall, ev = time_gpu(fn, args.steps, args.warmup)
     tflops = flops * args.steps / wall / 1e12
-    per_launch = ev / args.steps
+
+    # the dominant kernel alone: with the pre-pass switched off the grouped GEMM re-uses the
+    # quadrant sums the calls above left in the workspace
+    kernel_s, prepass_s = ev / args.steps, 0.0
+    staged = levels == 1 and algo != "classic" and nbytes > 0
+    if staged:
+        lib.sthip_debug_set_stages(2)
+        _, ev_k = time_gpu(fn, args.steps, 3)
+        lib.sthip_debug_set_stages(1)
+        _, ev_p = time_gpu(fn, args.steps, 3)
+        lib.sthip_debug_set_stages(3)
+        kernel_s, prepass_s = ev_k / args.steps, ev_p / args.steps
+        fn()   # leave `out` holding a complete result for the error figures below
 
     ref_out = torch.empty_like(out)
     wall_b, ev_b = time_gpu(lambda: torch.matmul(Ag, Bg, out=ref_out), args.steps, args.warmup)
@@ -153,21 +203,25 @@ def main():
     del exact, mine
 
     peak = PEAK_TFLOPS[DT_NAME[dtype]]
-    achieved = flops / per_launch / 1e12
+    achieved = flops / kernel_s / 1e12
+    executed = (7.0 / 8.0) ** (levels if algo != "classic" else 0)
     result = {
         "metric": "effective TFLOP/s (2MNK/t) at 8192^2 bf16; ratio vs hipBLASLt GEMM",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": DT_NAME[dtype], "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "M": M, "N": N, "K": K, "algo": algo, "levels": levels,
-                   "accumulate": "fp32", "aggregate": "fp32", "out_dtype": DT_NAME[dtype]},
+                   "accumulate": "fp32", "aggregate": "fp32", "out_dtype": DT_NAME[dtype],
+                   "workspace_bytes": nbytes},
         "hipblaslt_tflops": round(blas_tflops, 2), "ratio_vs_hipblaslt": round(tflops / blas_tflops, 4),
         "hipblaslt_ms": round(wall_b / args.steps * 1e3, 4),
+        "mfma_peak_frac": round(tflops / peak, 4),
         "rel_fro_err_vs_fp64": err64, "hipblaslt_rel_fro_err_vs_fp64": err_blas,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel_ms": round(per_launch * 1e3, 4),
-                     "executed_mfma_tflops": round(achieved * (7.0 / 8.0) ** (levels if algo != "classic" else 0), 2)},
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload),
+                     "kernel": "gemm3_kernel (grouped GEMM, 256x128 tiles)" if staged else "whole call",
+                     "kernel_ms": round(kernel_s * 1e3, 4), "prepass_ms": round(prepass_s * 1e3, 4),
+                     "flops_per_launch": flops, "executed_mfma_tflops": round(achieved * executed, 2)},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(A, B, max(levels, 1), dtype, algo)

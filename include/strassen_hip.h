@@ -47,9 +47,15 @@ enum sthip_algo {
  * each (so NN / NT / TN / TT all work without copies).  in_dtype is the element type of A
  * and B; out_dtype is that of C and must equal in_dtype or be STHIP_F32.  Products
  * accumulate in fp32, operand sums are formed in fp32 and rounded once to in_dtype, the
- * recombination is done in fp32.  levels = 1 runs one fused launch and needs no
- * workspace; levels >= 2 recurses on the host and needs sthip_workspace_bytes().  Sizes
- * that are not multiples of 2^levels behave as if zero padded.
+ * recombination is done in fp32.  Sizes that are not multiples of 2^levels behave as if
+ * zero padded.
+ *
+ * levels = 1 needs no workspace: one fused launch forms the quadrant sums in registers on
+ * the way from global memory to LDS.  Given sthip_workspace_bytes() of workspace, 16-bit
+ * problems whose half-size blocks are multiples of the tile (128 x 128 x 64) take the faster
+ * pipelined path instead: the ten quadrant sums are written once, then one grouped-GEMM
+ * launch runs the seven products and recombines them in registers.  levels >= 2 recurses on
+ * the host (sums and products of the upper levels in workspace) and requires the workspace.
  *
  * Replaces: _strassen_base (fixed_strassen.py:11-57, fixed_strassen_fp32_agg.py:12-56),
  * strassen_matmul_n_layers (fixed_strassen.py:59-126, fixed_strassen_fp32_agg.py:58-125),
@@ -62,7 +68,8 @@ int sthip_gemm(const void* A, const void* B, void* C,
                int in_dtype, int out_dtype, int algo, int levels, int accumulate,
                void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of device workspace sthip_gemm needs for this problem (0 when levels <= 1). */
+/* Bytes of device workspace sthip_gemm can use for this problem: optional for levels = 1 (0 if
+ * the pipelined path does not apply), required for levels >= 2.  Must be 256-byte aligned. */
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K,
                              int in_dtype, int out_dtype, int algo, int levels);
 
@@ -105,6 +112,13 @@ int sthip_version(void);
  * device memory).  Used by the tests to pin the lane mapping the kernels rely on.  No
  * counterpart in the reference. */
 int sthip_debug_transpose_read(void* out, void* stream);
+
+/* Profiling aid: selects which stages of the pipelined one-level path later calls run
+ * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM; default 3) and returns the previous
+ * mask.  With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so
+ * the dominant kernel can be timed alone.  Process-wide; not for production calls.  No
+ * counterpart in the reference. */
+int sthip_debug_set_stages(int mask);
 
 #ifdef __cplusplus
 }

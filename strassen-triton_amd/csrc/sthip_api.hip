@@ -12,6 +12,9 @@
 namespace sthip {
 
 static thread_local char g_err[512] = "";
+// Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM.
+// Only the profiling hook sthip_debug_set_stages changes it.
+static int g_stages = 3;
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -162,7 +165,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
         const int nout = algo == STHIP_STRASSEN ? 5 : 4;
-        for (int side = 0; side < 2; ++side) {
+        for (int side = 0; side < 2 && (g_stages & 1); ++side) {
             ComboParams cp;
             memset(&cp, 0, sizeof(cp));
             const bool kc = side == 0 ? a_kc : b_kc;
@@ -216,6 +219,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
         }
     }
+    if (!(g_stages & 2)) return STHIP_OK;
     // Fixed tile table: 256 x 128 tiles (less global->LDS traffic per flop) when A is contiguous
     // along k, the block height allows it and there is a tile for every one of the 256 CUs;
     // 128 x 128 tiles otherwise.
@@ -583,6 +587,12 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
         return check_launch("add_bias");
     }
     return STHIP_OK;
+}
+
+int sthip_debug_set_stages(int mask) {
+    const int old = g_stages;
+    g_stages = mask & 3;
+    return old;
 }
 
 const char* sthip_last_error(void) { return g_err; }

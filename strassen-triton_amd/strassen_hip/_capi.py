@@ -26,6 +26,7 @@ SIGNATURES = {
     "sthip_last_error": (ctypes.c_char_p, []),
     "sthip_version": (_int, []),
     "sthip_debug_transpose_read": (_int, [_vp, _vp]),
+    "sthip_debug_set_stages": (_int, [_int]),
 }
 
 _lib = None

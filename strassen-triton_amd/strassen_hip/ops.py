@@ -57,8 +57,20 @@ def _workspace(nbytes: int, device) -> tuple[torch.Tensor | None, int]:
     return ws, ws.data_ptr()
 
 
+def workspace_bytes(A: torch.Tensor, B: torch.Tensor, *, algo="strassen", levels: int = 1,
+                    out_dtype: torch.dtype | None = None) -> int:
+    """Bytes of scratch gemm(A, B, ...) would allocate; pass a uint8 tensor of at least that size
+    as `workspace=` to re-use one allocation across calls."""
+    algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    batch = A.shape[0] if A.dim() == 3 else 1
+    dt = _dtype_code(A.dtype)
+    return _capi.load().sthip_workspace_bytes(batch, A.shape[-2], B.shape[-1], A.shape[-1], dt,
+                                              _dtype_code(out_dtype or A.dtype), algo, levels)
+
+
 def gemm(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor | None = None, *, algo="strassen",
-         levels: int = 1, accumulate: bool = False, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+         levels: int = 1, accumulate: bool = False, out_dtype: torch.dtype | None = None,
+         workspace: torch.Tensor | None = None) -> torch.Tensor:
     """out (+)= A @ B through sthip_gemm.  A: (b,) M x K, B: (b,) K x N, same dtype."""
     _require_gpu(A, B)
     lib = _capi.load()
@@ -83,7 +95,12 @@ def gemm(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor | None = None, *, a
     out_dt = _dtype_code(out.dtype)
     A, B = _unit_stride(A), _unit_stride(B)
     nbytes = lib.sthip_workspace_bytes(batch, M, N, K, in_dt, out_dt, algo, levels)
-    ws, ws_ptr = _workspace(nbytes, A.device)
+    if workspace is not None and nbytes > 0:
+        if not workspace.is_cuda or workspace.dtype != torch.uint8 or workspace.numel() < nbytes:
+            raise ValueError(f"workspace must be a uint8 GPU tensor of at least {nbytes} bytes")
+        ws, ws_ptr = workspace, workspace.data_ptr()
+    else:
+        ws, ws_ptr = _workspace(nbytes, A.device)
     with torch.cuda.device(A.device):
         _capi.check(lib.sthip_gemm(A.data_ptr(), B.data_ptr(), out.data_ptr(), batch, M, N, K,
                                    _strides3(A), _strides3(B), _strides3(out), in_dt, out_dt, algo, levels,
