@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "../../include/strassen_hip.h"
@@ -60,6 +61,25 @@ static const LaunchTable3* table3_for(int dt, int algo) {
         case 6: return &kLaunch3_2_0; case 7: return &kLaunch3_2_1; case 8: return &kLaunch3_2_2;
     }
     return nullptr;
+}
+
+static const LaunchTable3* table4_for(int dt, int algo) {
+    switch (dt * 3 + algo) {
+        case 3: return &kLaunch4_1_0; case 4: return &kLaunch4_1_1; case 5: return &kLaunch4_1_2;
+        case 6: return &kLaunch4_2_0; case 7: return &kLaunch4_2_1; case 8: return &kLaunch4_2_2;
+    }
+    return nullptr;
+}
+
+// STHIP_FORCE_TILE=128x128 | 256x128 | 256x256 overrides the tile table where the shape allows
+// the forced tile (tuning and test aid); unset or anything else = automatic.
+static int forced_tile() {
+    const char* e = getenv("STHIP_FORCE_TILE");
+    if (!e) return 0;
+    if (!strcmp(e, "128x128")) return 2;
+    if (!strcmp(e, "256x128")) return 3;
+    if (!strcmp(e, "256x256")) return 4;
+    return 0;
 }
 
 static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -126,10 +146,11 @@ static const signed char kStrB[5][4] = {{0, 1, 0, -1}, {-1, 0, 1, 0}, {1, 0, 0, 
 static const signed char kWinA[4][4] = {{0, 0, 1, 1}, {-1, 0, 1, 1}, {1, 0, -1, 0}, {1, 1, -1, -1}};
 static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0, 1}, {-1, 1, 1, -1}};
 
-// Workspace of the pipelined path per problem: five sums per operand plus one fp32 tile per
-// workgroup for the accumulator the 256 x 128 Strassen kernel parks (Mh x Nh floats in all).
+// Workspace of the pipelined path per problem: five sums per operand plus fp32 slabs for the
+// accumulator tiles the large-tile kernels park (one tile per workgroup for 256 x 128, three
+// for 256 x 256: at most 3 x Mh x Nh floats).
 static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
-    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + align256(Mh * Nh * 4));
+    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + 3 * align256(Mh * Nh * 4));
 }
 
 static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
@@ -220,13 +241,31 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         }
     }
     if (!(g_stages & 2)) return STHIP_OK;
-    // Fixed tile table: 256 x 128 tiles (less global->LDS traffic per flop) when A is contiguous
-    // along k, the block height allows it and there is a tile for every one of the 256 CUs;
-    // 128 x 128 tiles otherwise.
+    // Fixed tile table.  Bytes moved L2 -> LDS per flop go with 1/BM + 1/BN, so the largest tile
+    // that still gives every CU work wins: 256 x 256 (one accumulator in registers), then
+    // 256 x 128 (two in registers, one parked), then 128 x 128 (three in registers).  The large
+    // tiles need A contiguous along k.
     hipError_t e;
     const LaunchTable3* t3 = table3_for(dt, algo);
-    const int64_t big_tiles = (Mh / kBM3) * (Nh / kBN3) * batch;
-    if (a_kc && Mh % kBM3 == 0 && t3 && big_tiles >= 256) {   // at least one 256 x 128 tile per CU
+    const LaunchTable3* t4 = table4_for(dt, algo);
+    const int force = forced_tile();
+    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4;
+    const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
+    const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch, tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
+    int pick = 2;
+    // 256 x 256 only for the classical product: with one accumulator in registers every chain of
+    // the Strassen / Winograd recombination is parked, and all CUs park at the same moment
+    // (64 MiB per event chip-wide) -- measured 1.59 ms against 1.04 ms for 256 x 128 at 8192^3.
+    if (can4 && tiles4 >= 224 && !split) pick = 4;
+    else if (can3 && tiles3 >= 256) pick = 3;
+    if (force == 4 && can4) pick = 4;
+    else if (force == 3 && can3) pick = 3;
+    else if (force == 2) pick = 2;
+    if (pick == 4) {
+        p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
+        p.group_m = 4;
+        e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+    } else if (pick == 3) {
         p.tiles_m = (int)(Mh / kBM3);
         p.group_m = 4;
         e = t3->fn[b_kc ? 1 : 0](p, (int)batch, stream);

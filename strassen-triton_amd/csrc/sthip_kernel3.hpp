@@ -217,8 +217,10 @@ struct Pipe3 {
 // Store (or accumulate into) this wave's 128 x 64 part of C block `quad`; (row, col) is the
 // wave tile's origin inside the block.  Lane l of MFMA tile (i, j) holds m = l%32 and, in
 // registers 4g..4g+3, n = 8g + 4*(l/32) + 0..3, so every store is 8 (or 16) contiguous bytes.
-template <class T>
-__device__ __forceinline__ void store_tile3(const Acc3& acc, const Gemm2Params& P, char* Cb, int quad, int row, int col) {
+// With PLUS the stored value is acc + plus, formed on the fly (neither tile is modified).
+template <class T, bool PLUS = false>
+__device__ __forceinline__ void store_tile3(const Acc3& acc, const Gemm2Params& P, char* Cb, int quad, int row, int col,
+                                            const Acc3& plus) {
     const int lane = threadIdx.x & 63;
     const int esz = P.out_f32 ? 4 : 2;
     const int m0 = (quad >> 1) * P.Mh + row + (lane & 31);
@@ -231,7 +233,7 @@ __device__ __forceinline__ void store_tile3(const Acc3& acc, const Gemm2Params& 
             for (int g = 0; g < 4; ++g) {
                 float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc.t[i][j][4 * g + e];
+                for (int e = 0; e < 4; ++e) v[e] = PLUS ? acc.t[i][j][4 * g + e] + plus.t[i][j][4 * g + e] : acc.t[i][j][4 * g + e];
                 char* dst = Cb + ((int64_t)(m0 + i * 32) * P.c_rs + (n0 + j * 32 + 8 * g)) * esz;
                 if (P.out_f32) {
                     f32x4* d = reinterpret_cast<f32x4*>(dst);
@@ -317,7 +319,7 @@ __global__ void __launch_bounds__(kThreads3) gemm3_kernel(const Gemm2Params P) {
     pipe.ld.point_at_segment();
     pipe.start();
 
-#define EMIT3(acc, quad) store_tile3<T>(acc, P, Cb, quad, tile_m + pipe.wm, tile_n + pipe.wn)
+#define EMIT3(acc, quad) store_tile3<T, false>(acc, P, Cb, quad, tile_m + pipe.wm, tile_n + pipe.wn, acc)
     enum { Q11 = 0, Q12 = 1, Q21 = 2, Q22 = 3 };
     if constexpr (ALGO == ALGO_CLASSIC) {
         Acc3 x;
@@ -355,25 +357,25 @@ __global__ void __launch_bounds__(kThreads3) gemm3_kernel(const Gemm2Params P) {
         park_add(x, slab);
         EMIT3(x, Q11);         // C11 = M1 + M4 - M5 + M7
     } else {
-        // segment order P1 P2 P6 P7 P5 P3 (-P4)
-        Acc3 x, y, z;
+        // segment order P1 P2 P6 P7 P5 P3 (-P4); two tiles in registers, U2 parked once
+        float* slab = P.park + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (kBM3 * kBN3);
+        Acc3 x, y;
         x.zero();
-        pipe.run(x, KT);   // P1
+        pipe.run(x, KT);       // P1
         y = x;
-        pipe.run(x, KT);   // + P2 -> C11
-        EMIT3(x, Q11);
-        pipe.run(y, KT);   // + P6 -> U2
-        z = y;
-        pipe.run(y, KT);   // + P7 -> U3
+        pipe.run(x, KT);       // + P2
+        EMIT3(x, Q11);         // C11 = P1 + P2
+        pipe.run(y, KT);       // + P6 -> U2
+        park_store(y, slab);
+        pipe.run(y, KT);       // + P7 -> U3
         x.zero();
-        pipe.run(x, KT);   // P5
-        z.add(x);          // U4
-        x.add(y);          // C22
-        EMIT3(x, Q22);
-        pipe.run(z, KT);   // + P3 -> C12
-        EMIT3(z, Q12);
-        pipe.run(y, KT);   // + A22 (-T4) -> C21
-        EMIT3(y, Q21);
+        pipe.run(x, KT);       // P5
+        store_tile3<T, true>(x, P, Cb, Q22, tile_m + pipe.wm, tile_n + pipe.wn, y);   // C22 = U3 + P5
+        park_add(x, slab);     // U4 = U2 + P5
+        pipe.run(x, KT);       // + P3
+        EMIT3(x, Q12);         // C12 = U4 + P3
+        pipe.run(y, KT);       // + A22 (-T4)
+        EMIT3(y, Q21);         // C21 = U3 - P4
     }
 #undef EMIT3
 }

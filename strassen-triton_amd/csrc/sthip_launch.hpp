@@ -4,6 +4,7 @@
 #include "sthip_kernel.hpp"
 #include "sthip_kernel2.hpp"
 #include "sthip_kernel3.hpp"
+#include "sthip_kernel4.hpp"
 
 namespace sthip {
 
@@ -84,6 +85,29 @@ hipError_t launch_gemm3(const Gemm2Params& p, int batch, hipStream_t stream) {
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads3), kSmemBytes3, stream, p);
+    return hipGetLastError();
+}
+
+// 256 x 256 kernel (16-bit operands, A contiguous along k): tables indexed [b_kc].
+#define STHIP_DECLARE_TABLE4(T, A) extern const LaunchTable3 kLaunch4_##T##_##A;
+STHIP_DECLARE_TABLE4(1, 0) STHIP_DECLARE_TABLE4(1, 1) STHIP_DECLARE_TABLE4(1, 2)
+STHIP_DECLARE_TABLE4(2, 0) STHIP_DECLARE_TABLE4(2, 1) STHIP_DECLARE_TABLE4(2, 2)
+#undef STHIP_DECLARE_TABLE4
+
+template <class T, int ALGO, bool B_KC>
+hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
+    auto kern = gemm4_kernel<T, ALGO, B_KC>;
+    static bool opted[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && !opted[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes4);
+        if (e != hipSuccess) return e;
+        opted[dev] = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, p);
     return hipGetLastError();
 }
 

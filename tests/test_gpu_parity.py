@@ -228,3 +228,26 @@ def test_autograd_matmul(hip):
     G = _ints((256, 384), 33, -1, 1).cuda()
     hip.matmul(A, B).backward(G)
     assert torch.equal(A.grad, G @ B.detach().T) and torch.equal(B.grad, A.detach().T @ G)
+
+
+@pytest.mark.parametrize("tile", ["128x128", "256x128", "256x256"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
+@pytest.mark.parametrize("tb", [False, True])
+def test_every_pipelined_tile_exact(hip, monkeypatch, tile, dtype, algo, tb):
+    """The tile table picks by size; force each pipelined kernel on a small aligned problem so
+    that all of them are checked bit for bit (integer inputs), with two batch entries, and again
+    in accumulate mode with an fp32 result."""
+    monkeypatch.setenv("STHIP_FORCE_TILE", tile)
+    b, M, N, K = 2, 1024, 1024, 512
+    A, B = _ints((b, M, K), 51, -1, 1, dtype), _ints((b, K, N), 52, -1, 1, dtype)
+    want = A.double() @ B.double()
+    Bg = _layout(B, tb)
+    C = hip.gemm(A.cuda(), Bg, algo=algo, levels=1, out_dtype=torch.float32)
+    assert torch.equal(C.cpu().double(), want)
+    C0 = _ints((b, M, N), 53, -3, 3, torch.float32)
+    Cacc = C0.clone().cuda()
+    hip.gemm(A.cuda(), Bg, out=Cacc, algo=algo, levels=1, accumulate=True)
+    assert torch.equal(Cacc.cpu().double(), C0.double() + want)
+    Cn = hip.gemm(A[0, :, :128].contiguous().cuda(), _layout(B[0, :128], tb), algo=algo, levels=1)   # |C| <= 128: exact in 16 bit
+    assert Cn.dtype == dtype and torch.equal(Cn.cpu().double(), A[0, :, :128].double() @ B[0, :128].double())
