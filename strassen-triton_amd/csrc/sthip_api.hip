@@ -429,6 +429,75 @@ static int check_launch(const char* what) {
     return STHIP_OK;
 }
 
+// All quadrant sums of one operand in one launch (see quad_combos_kernel).  X is the operand,
+// (r_blk, c_blk) the block size in its logical (row, col) indexing; outputs are dense blocks in
+// the storage orientation of X, `out_stride` bytes apart.
+static bool combos_ok(View X, int64_t r_blk, int64_t c_blk) {
+    if (!aligned_to(X.p, 16)) return false;
+    if (X.cs == 1) return c_blk % 8 == 0 && X.rs % 8 == 0;
+    if (X.rs == 1) return r_blk % 8 == 0 && X.cs % 8 == 0;
+    return false;
+}
+
+static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, size_t out_stride, int nout,
+                      const signed char (*coef)[4], hipStream_t stream) {
+    ComboParams cp;
+    memset(&cp, 0, sizeof(cp));
+    const bool row_major = X.cs == 1;
+    for (int q = 0; q < 4; ++q)
+        cp.q[q] = X.p + ((int64_t)(q >> 1) * r_blk * X.rs + (int64_t)(q & 1) * c_blk * X.cs) * 2;
+    for (int o = 0; o < nout; ++o) {
+        cp.out[o] = out + (size_t)o * out_stride;
+        for (int q = 0; q < 4; ++q) cp.coef[o][q] = coef[o][q];
+    }
+    const int64_t rows = row_major ? r_blk : c_blk, cols = row_major ? c_blk : r_blk;   // storage order
+    cp.ld_in = row_major ? X.rs : X.cs;
+    cp.ld_out = cols;
+    cp.nout = nout; cp.rows = (int)rows; cp.chunks_per_row = (int)(cols / 8);
+    const int64_t n = rows * (cols / 8);
+    if (n == 0) return STHIP_OK;
+    dim3 grid((unsigned)ceil_div(n, 256), 1);
+    if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, stream, cp);
+    else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, stream, cp);
+    return check_launch("quad_combos");
+}
+
+// Vector form of recombine_kernel: four consecutive columns per thread (nh % 4 == 0, C with unit
+// column stride, 4-element aligned rows, M = 2 mh, N = 2 nh).
+template <class TO>
+__global__ void recombine_vec_kernel(char* C, int64_t c_rs, const float* Mbuf, int64_t mstride, int mh, int nh, int accumulate) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int nq = nh / 4;
+    if (idx >= (int64_t)mh * nq) return;
+    const int i = (int)(idx / nq), j = (int)(idx % nq) * 4;
+    f32x4 m[7];
+#pragma unroll
+    for (int q = 0; q < 7; ++q) m[q] = *reinterpret_cast<const f32x4*>(Mbuf + q * mstride + (int64_t)i * nh + j);
+    const f32x4 out[4] = {m[0] + m[3] - m[4] + m[6], m[2] + m[4], m[1] + m[3], m[0] - m[1] + m[2] + m[5]};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int64_t off = (int64_t)(i + (q >> 1) * mh) * c_rs + (j + (q & 1) * nh);
+        f32x4 v = out[q];
+        if constexpr (sizeof(TO) == 4) {
+            f32x4* d = reinterpret_cast<f32x4*>(C) + off / 4;
+            if (accumulate) v += *d;
+            *d = v;
+        } else {
+            u32x2* d = reinterpret_cast<u32x2*>(C + off * 2);
+            if (accumulate) {
+                const u32x2 old = *d;
+                const uint32_t w0 = old[0], w1 = old[1];
+                if constexpr (__is_same(TO, bf16_t)) { v[0] += bf16lo(w0); v[1] += bf16hi(w0); v[2] += bf16lo(w1); v[3] += bf16hi(w1); }
+                else { const f16x2 h0 = as_f16x2(w0), h1 = as_f16x2(w1); v[0] += (float)h0[0]; v[1] += (float)h0[1]; v[2] += (float)h1[0]; v[3] += (float)h1[1]; }
+            }
+            u32x2 o;
+            if constexpr (__is_same(TO, bf16_t)) { o[0] = pack_bf16(v[0], v[1]); o[1] = pack_bf16(v[2], v[3]); }
+            else { o[0] = pack_f16(v[0], v[1]); o[1] = pack_f16(v[2], v[3]); }
+            *d = o;
+        }
+    }
+}
+
 static int block_sum(int dt, char* dst, View X, int ra, int ca, int rb, int cb, int sign,
                      int64_t rows, int64_t cols, int64_t lim_r, int64_t lim_c, hipStream_t s) {
     const int64_t n = rows * cols;
@@ -444,6 +513,15 @@ static int recombine(int out_dt, char* C, int64_t c_rs, int64_t c_cs, const floa
                      int64_t mh, int64_t nh, int64_t M, int64_t N, bool accumulate, hipStream_t s) {
     const int64_t n = mh * nh;
     if (n == 0) return STHIP_OK;
+    const size_t oes = out_dt == STHIP_F32 ? 4 : 2;
+    if (c_cs == 1 && nh % 4 == 0 && c_rs % 4 == 0 && M == 2 * mh && N == 2 * nh && aligned_to(C, 4 * oes) && mstride % 4 == 0) {
+        const unsigned vb = (unsigned)ceil_div(n / 4, 256);
+        const int acc = accumulate ? 1 : 0;
+        if (out_dt == STHIP_F32) hipLaunchKernelGGL(recombine_vec_kernel<float>, dim3(vb), dim3(256), 0, s, C, c_rs, Mbuf, mstride, (int)mh, (int)nh, acc);
+        else if (out_dt == STHIP_F16) hipLaunchKernelGGL(recombine_vec_kernel<f16_t>, dim3(vb), dim3(256), 0, s, C, c_rs, Mbuf, mstride, (int)mh, (int)nh, acc);
+        else hipLaunchKernelGGL(recombine_vec_kernel<bf16_t>, dim3(vb), dim3(256), 0, s, C, c_rs, Mbuf, mstride, (int)mh, (int)nh, acc);
+        return check_launch("recombine_vec");
+    }
     const unsigned blocks = (unsigned)ceil_div(n, 256);
 #define GO(T) hipLaunchKernelGGL(recombine_kernel<T>, dim3(blocks), dim3(256), 0, s, C, c_rs, c_cs, Mbuf, mstride, (int)mh, (int)nh, (int)M, (int)N, accumulate ? 1 : 0)
     if (out_dt == STHIP_F32) GO(float); else if (out_dt == STHIP_F16) GO(f16_t); else GO(bf16_t);
@@ -463,7 +541,7 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
     if (levels <= 0) return 0;
     if (levels == 1) return fast_shape(dt, mh, nh, kh) ? prepass_bytes(1, mh, nh, kh) : 0;
     const size_t es = elem_size(dt);
-    return align256(mh * kh * es) + align256(kh * nh * es) + 7 * align256(mh * nh * 4) +
+    return 5 * (align256(mh * kh * es) + align256(kh * nh * es)) + 7 * align256(mh * nh * 4) +
            workspace_for(mh, nh, kh, dt, levels - 1);
 }
 
@@ -484,22 +562,37 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
 
     const size_t es = elem_size(dt);
     const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es), m_b = align256(mh * nh * 4);
-    const size_t need = sa_b + sb_b + 7 * m_b;
+    const size_t need = 5 * (sa_b + sb_b) + 7 * m_b;
     if (!ws || ws_bytes < need) return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, need);
     char* SA = ws;
-    char* SB = ws + sa_b;
-    char* Mbuf = ws + sa_b + sb_b;
+    char* SB = ws + 5 * sa_b;
+    char* Mbuf = ws + 5 * (sa_b + sb_b);
     char* child_ws = ws + need;
     const size_t child_bytes = ws_bytes - need;
+
+    // Whole, aligned 16-bit problems: all five sums of each operand in one bandwidth-bound launch.
+    const bool whole = M == Mp && N == Np && K == Kp;
+    const bool vec = dt != STHIP_F32 && whole && combos_ok(A, mh, kh) && combos_ok(B, kh, nh);
+    if (vec) {
+        int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, stream);
+        if (rc) return rc;
+        rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, stream);
+        if (rc) return rc;
+    }
+    // sums by product M1..M7 as indices into the outputs of kStrA / kStrB (-1 = a raw block)
+    static const int kSumA[7] = {2, 1, -1, -1, 0, 4, 3};
+    static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
 
     for (int q = 0; q < 7; ++q) {
         const Term ta = kATerms[q], tb = kBTerms[q];
         View a, b;
-        int64_t am = mh, ak = kh, bk = kh, bn = nh;   // logical extents of the operands handed down
         // A operand: a single block that lies fully inside A is used in place
         const int ara = (ta.a >> 1) * (int)mh, aca = (ta.a & 1) * (int)kh;
         if (ta.sign == 0 && ara + mh <= M && aca + kh <= K) {
             a = {A.p + ((int64_t)ara * A.rs + (int64_t)aca * A.cs) * (int64_t)es, A.rs, A.cs};
+        } else if (vec) {
+            const char* p = SA + (size_t)kSumA[q] * sa_b;   // dense, in A's storage orientation
+            a = A.cs == 1 ? View{p, kh, 1} : View{p, 1, mh};
         } else {
             int rc = block_sum(dt, SA, A, ara, aca, (ta.b >> 1) * (int)mh, (ta.b & 1) * (int)kh, ta.sign, mh, kh, M, K, stream);
             if (rc) return rc;
@@ -508,14 +601,16 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         const int bra = (tb.a >> 1) * (int)kh, bca = (tb.a & 1) * (int)nh;
         if (tb.sign == 0 && bra + kh <= K && bca + nh <= N) {
             b = {B.p + ((int64_t)bra * B.rs + (int64_t)bca * B.cs) * (int64_t)es, B.rs, B.cs};
+        } else if (vec) {
+            const char* p = SB + (size_t)kSumB[q] * sb_b;
+            b = B.cs == 1 ? View{p, nh, 1} : View{p, 1, kh};
         } else {
             int rc = block_sum(dt, SB, B, bra, bca, (tb.b >> 1) * (int)kh, (tb.b & 1) * (int)nh, tb.sign, kh, nh, K, N, stream);
             if (rc) return rc;
             b = {SB, nh, 1};
         }
-        int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, am, bn, ak, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
+        int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, mh, nh, kh, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
                           false, child_ws, child_bytes, stream);
-        (void)bk;
         if (rc) return rc;
     }
     return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, stream);

@@ -52,11 +52,12 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
-    # Two levels: one S_A, one S_B and seven fp32 M buffers of half size, plus the leaf's sums.
+    # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace.
+    upper = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
-    assert two == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4 + sums(256)
+    assert two == upper(512) + sums(256)
     three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
-    assert three == 2 * 512 * 512 * 2 + 7 * 512 * 512 * 4 + 2 * 256 * 256 * 2 + 7 * 256 * 256 * 4 + sums(128)
+    assert three == upper(512) + upper(256) + sums(128)
 
 
 def test_reference_recursion_depth():
