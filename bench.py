@@ -180,15 +180,17 @@ def main():
 
     # the dominant kernel alone: with the pre-pass switched off the grouped GEMM re-uses the
     # quadrant sums the calls above left in the workspace
-    kernel_s, prepass_s = ev / args.steps, 0.0
+    kernel_s, prepass_s, recombine_s = ev / args.steps, 0.0, 0.0
     staged = levels == 1 and algo != "classic" and nbytes > 0
     if staged:
         lib.sthip_debug_set_stages(2)
         _, ev_k = time_gpu(fn, args.steps, 3)
         lib.sthip_debug_set_stages(1)
         _, ev_p = time_gpu(fn, args.steps, 3)
-        lib.sthip_debug_set_stages(3)
-        kernel_s, prepass_s = ev_k / args.steps, ev_p / args.steps
+        lib.sthip_debug_set_stages(4)
+        _, ev_r = time_gpu(fn, args.steps, 3)
+        lib.sthip_debug_set_stages(7)
+        kernel_s, prepass_s, recombine_s = ev_k / args.steps, ev_p / args.steps, ev_r / args.steps
         fn()   # leave `out` holding a complete result for the error figures below
 
     ref_out = torch.empty_like(out)
@@ -219,8 +221,9 @@ def main():
         "rel_fro_err_vs_fp64": err64, "hipblaslt_rel_fro_err_vs_fp64": err_blas,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload),
-                     "kernel": "gemm3_kernel (grouped GEMM, 256x128 tiles)" if staged else "whole call",
+                     "kernel": "grouped GEMM launch of the call (stage mask 2)" if staged else "whole call",
                      "kernel_ms": round(kernel_s * 1e3, 4), "prepass_ms": round(prepass_s * 1e3, 4),
+                     "recombine_ms": round(recombine_s * 1e3, 4),
                      "flops_per_launch": flops, "executed_mfma_tflops": round(achieved * executed, 2)},
     }
     if not args.no_cpu:

@@ -53,8 +53,11 @@ enum sthip_algo {
  * levels = 1 needs no workspace: one fused launch forms the quadrant sums in registers on
  * the way from global memory to LDS.  Given sthip_workspace_bytes() of workspace, 16-bit
  * problems whose half-size blocks are multiples of the tile (128 x 128 x 64) take the faster
- * pipelined path instead: the ten quadrant sums are written once, then one grouped-GEMM
- * launch runs the seven products and recombines them in registers.  levels >= 2 recurses on
+ * pipelined path instead: the quadrant sums are written once, then one grouped-GEMM launch
+ * runs the seven products.  Large problems (half-size blocks multiples of 256, result in the
+ * operand type) use 256 x 256 tiles, round each product once to the operand type as the
+ * reference's mm does, and recombine in a third pass in fp32; the others recombine in
+ * registers without that rounding.  levels >= 2 recurses on
  * the host (sums and products of the upper levels in workspace) and requires the workspace.
  *
  * Replaces: _strassen_base (fixed_strassen.py:11-57, fixed_strassen_fp32_agg.py:12-56),
@@ -114,10 +117,10 @@ int sthip_version(void);
 int sthip_debug_transpose_read(void* out, void* stream);
 
 /* Profiling aid: selects which stages of the pipelined one-level path later calls run
- * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM; default 3) and returns the previous
- * mask.  With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so
- * the dominant kernel can be timed alone.  Process-wide; not for production calls.  No
- * counterpart in the reference. */
+ * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM, bit 2 = recombination pass of the
+ * 256 x 256 path; default 7) and returns the previous mask.  With mask 2 the GEMM re-uses the
+ * sums a previous call left in the same workspace, so the dominant kernel can be timed alone.
+ * Process-wide; not for production calls.  No counterpart in the reference. */
 int sthip_debug_set_stages(int mask);
 
 #ifdef __cplusplus

@@ -42,8 +42,7 @@ def _units():
         for a in range(3):
             units.append((f"sthip_inst3_{t}_{a}.o", "sthip_inst3.hip",
                           [f"-DSTHIP_INST_TYPE={t}", f"-DSTHIP_INST_ALGO={a}"]))
-            units.append((f"sthip_inst4_{t}_{a}.o", "sthip_inst4.hip",
-                          [f"-DSTHIP_INST_TYPE={t}", f"-DSTHIP_INST_ALGO={a}"]))
+        units.append((f"sthip_inst4_{t}.o", "sthip_inst4.hip", [f"-DSTHIP_INST_TYPE={t}"]))
     return units
 
 

@@ -15,7 +15,7 @@ namespace sthip {
 static thread_local char g_err[512] = "";
 // Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM.
 // Only the profiling hook sthip_debug_set_stages changes it.
-static int g_stages = 3;
+static int g_stages = 7;
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -63,12 +63,8 @@ static const LaunchTable3* table3_for(int dt, int algo) {
     return nullptr;
 }
 
-static const LaunchTable3* table4_for(int dt, int algo) {
-    switch (dt * 3 + algo) {
-        case 3: return &kLaunch4_1_0; case 4: return &kLaunch4_1_1; case 5: return &kLaunch4_1_2;
-        case 6: return &kLaunch4_2_0; case 7: return &kLaunch4_2_1; case 8: return &kLaunch4_2_2;
-    }
-    return nullptr;
+static const LaunchTable3* table4_for(int dt) {
+    return dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
 }
 
 // STHIP_FORCE_TILE=128x128 | 256x128 | 256x256 overrides the tile table where the shape allows
@@ -146,11 +142,79 @@ static const signed char kStrB[5][4] = {{0, 1, 0, -1}, {-1, 0, 1, 0}, {1, 0, 0, 
 static const signed char kWinA[4][4] = {{0, 0, 1, 1}, {-1, 0, 1, 1}, {1, 0, -1, 0}, {1, 1, -1, -1}};
 static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0, 1}, {-1, 1, 1, -1}};
 
-// Workspace of the pipelined path per problem: five sums per operand plus fp32 slabs for the
-// accumulator tiles the large-tile kernels park (one tile per workgroup for 256 x 128, three
-// for 256 x 256: at most 3 x Mh x Nh floats).
+// Workspace of the pipelined path per problem: five sums per operand, then a region that is
+// either the seven 16-bit products of the 256 x 256 grouped launch or the fp32 slabs in which
+// the 256 x 128 kernel parks one accumulator tile per workgroup (at most Mh x Nh floats).
+static size_t products_bytes(int64_t Mh, int64_t Nh) { return 7 * align256(Mh * Nh * 2); }
 static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
-    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + 3 * align256(Mh * Nh * 4));
+    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + products_bytes(Mh, Nh));
+}
+
+// Recombination of the seven 16-bit products of one level (kernel order: Strassen
+// M3 M6 M5 M7 M1 M2 M4, Winograd P1 P2 P6 P7 P5 P3 -P4) into the four quadrants of C: upcast,
+// add in fp32 in the reference's order (fixed_strassen_fp32_agg.py:44-53), round once.  One
+// thread per 16-byte chunk of a half-size row.
+struct Recombine16Params {
+    const void* prod;     // [batch][7][Mh x Nh]
+    void* C;
+    int64_t c_rs, c_bs;   // elements
+    int Mh, Nh, accumulate;
+};
+
+template <class T>
+__device__ __forceinline__ void unpack8(const u32x4 v, float* x) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if constexpr (__is_same(T, bf16_t)) { x[2 * w] = bf16lo(v[w]); x[2 * w + 1] = bf16hi(v[w]); }
+        else { const f16x2 h = as_f16x2(v[w]); x[2 * w] = (float)h[0]; x[2 * w + 1] = (float)h[1]; }
+    }
+}
+
+template <class T, int ALGO>
+__global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Params p) {
+    const int nq = p.Nh / 8;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.Mh * nq) return;
+    const int i = (int)(idx / nq), j = (int)(idx % nq) * 8;
+    const int64_t blk = (int64_t)p.Mh * p.Nh;
+    const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)blockIdx.y * 7 * blk + (int64_t)i * p.Nh + j) * 2;
+    float m[7][8];
+#pragma unroll
+    for (int q = 0; q < 7; ++q) unpack8<T>(*reinterpret_cast<const u32x4*>(src + q * blk * 2), m[q]);
+    float out[4][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        if constexpr (ALGO == STHIP_STRASSEN) {
+            out[0][e] = ((m[4][e] + m[6][e]) - m[2][e]) + m[3][e];   // C11 = M1 + M4 - M5 + M7
+            out[1][e] = m[0][e] + m[2][e];                           // C12 = M3 + M5
+            out[2][e] = m[5][e] + m[6][e];                           // C21 = M2 + M4
+            out[3][e] = ((m[4][e] - m[5][e]) + m[0][e]) + m[1][e];   // C22 = M1 - M2 + M3 + M6
+        } else {
+            const float u2 = m[0][e] + m[2][e], u3 = u2 + m[3][e], u4 = u2 + m[4][e];
+            out[0][e] = m[0][e] + m[1][e];                           // C11 = P1 + P2
+            out[1][e] = u4 + m[5][e];                                // C12 = U4 + P3
+            out[2][e] = u3 + m[6][e];                                // C21 = U3 - P4
+            out[3][e] = u3 + m[4][e];                                // C22 = U3 + P5
+        }
+    }
+    char* Cb = reinterpret_cast<char*>(p.C) + (int64_t)blockIdx.y * p.c_bs * 2;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        u32x4* d = reinterpret_cast<u32x4*>(Cb + ((int64_t)(i + (q >> 1) * p.Mh) * p.c_rs + (j + (q & 1) * p.Nh)) * 2);
+        if (p.accumulate) {
+            float old[8];
+            unpack8<T>(*d, old);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[q][e] += old[e];
+        }
+        u32x4 w;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if constexpr (__is_same(T, bf16_t)) w[k] = pack_bf16(out[q][2 * k], out[q][2 * k + 1]);
+            else w[k] = pack_f16(out[q][2 * k], out[q][2 * k + 1]);
+        }
+        *d = w;
+    }
 }
 
 static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
@@ -240,30 +304,55 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
         }
     }
-    if (!(g_stages & 2)) return STHIP_OK;
     // Fixed tile table.  Bytes moved L2 -> LDS per flop go with 1/BM + 1/BN, so the largest tile
-    // that still gives every CU work wins: 256 x 256 (one accumulator in registers), then
-    // 256 x 128 (two in registers, one parked), then 128 x 128 (three in registers).  The large
-    // tiles need A contiguous along k.
-    hipError_t e;
+    // that still gives every CU work wins.  256 x 256 holds one accumulator per wave and nothing
+    // else: a classical product runs on it directly, a Strassen / Winograd level runs its seven
+    // products on it as one grouped launch into 16-bit product matrices (the reference's own
+    // cast schedule) followed by the recombination pass.  256 x 128 (two accumulators in
+    // registers, one parked) and 128 x 128 (three in registers) recombine in registers and serve
+    // fp32 results and the sizes that are too small for the large tile.  The large tiles need A
+    // contiguous along k; the recombination pass needs 16-byte aligned rows of C.
+    hipError_t e = hipSuccess;
     const LaunchTable3* t3 = table3_for(dt, algo);
-    const LaunchTable3* t4 = table4_for(dt, algo);
+    const LaunchTable3* t4 = table4_for(dt);
     const int force = forced_tile();
-    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4;
+    const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
+    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && (!split || (!out_f32 && c_vec));
     const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
-    const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch, tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
+    const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch * (split ? 7 : 1);
+    const int64_t tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
     int pick = 2;
-    // 256 x 256 only for the classical product: with one accumulator in registers every chain of
-    // the Strassen / Winograd recombination is parked, and all CUs park at the same moment
-    // (64 MiB per event chip-wide) -- measured 1.59 ms against 1.04 ms for 256 x 128 at 8192^3.
-    if (can4 && tiles4 >= 224 && !split) pick = 4;
+    if (can4 && tiles4 >= (split ? 400 : 224)) pick = 4;
     else if (can3 && tiles3 >= 256) pick = 3;
     if (force == 4 && can4) pick = 4;
     else if (force == 3 && can3) pick = 3;
     else if (force == 2) pick = 2;
+    if (pick == 4 && split) {
+        Recombine16Params rp;
+        rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
+        rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
+        if (g_stages & 2) {
+            p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
+            p.out_f32 = 0; p.accumulate = 0; p.nprod = 7;
+            p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
+            p.group_m = 4;
+            e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+            if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+        }
+        if (g_stages & 4) {
+            dim3 grid((unsigned)ceil_div(Mh * (Nh / 8), 256), (unsigned)batch);
+#define GO(T, A) hipLaunchKernelGGL((recombine16_kernel<T, A>), grid, dim3(256), 0, stream, rp)
+            if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
+            else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
+#undef GO
+            return check_launch("recombine16");
+        }
+        return STHIP_OK;
+    }
+    if (!(g_stages & 2)) return STHIP_OK;
     if (pick == 4) {
         p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
-        p.group_m = 4;
+        p.group_m = 4; p.nprod = 1;
         e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
     } else if (pick == 3) {
         p.tiles_m = (int)(Mh / kBM3);
@@ -725,7 +814,7 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
 
 int sthip_debug_set_stages(int mask) {
     const int old = g_stages;
-    g_stages = mask & 3;
+    g_stages = mask & 7;
     return old;
 }
 

@@ -478,8 +478,7 @@ __device__ __forceinline__ void emit(const Acc& acc, const GemmParams& P, char* 
 // its own L2; renumber so that one XCD works on a contiguous run of tiles, then walk the
 // tile grid in groups of group_m tile-rows so that the run reuses A row-panels and B
 // column-panels out of that L2.
-__device__ __forceinline__ void tile_coords(const GemmParams& P, int& tm, int& tn) {
-    const int nb = gridDim.x, bid = blockIdx.x;
+__device__ __forceinline__ void tile_coords_in(const GemmParams& P, int bid, int nb, int& tm, int& tn) {
     const int per = nb / 8, rem = nb % 8;
     const int xcd = bid % 8, idx = bid / 8;
     const int logical = idx + (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per);
@@ -489,6 +488,9 @@ __device__ __forceinline__ void tile_coords(const GemmParams& P, int& tm, int& t
     const int gsz = min(P.tiles_m - first, P.group_m);
     tm = first + in % gsz;
     tn = in / gsz;
+}
+__device__ __forceinline__ void tile_coords(const GemmParams& P, int& tm, int& tn) {
+    tile_coords_in(P, (int)blockIdx.x, (int)gridDim.x, tm, tn);
 }
 
 template <class T, int ALGO, bool A_KC, bool B_KC, bool EDGE>

@@ -48,6 +48,8 @@ struct Gemm2Params {
     void* C;
     float* park;          // scratch for one parked accumulator tile per workgroup (256 x 128 kernel, Strassen)
     int64_t c_rs, c_bs;   // C is row-major with unit column stride
+    int64_t c_ps;         // 256 x 256 kernel: element stride between the outputs of consecutive products
+    int nprod;            // 256 x 256 kernel: products in this launch (1 = plain GEMM)
     int Mh, Nh, Kh;       // extent of one segment product
     int tiles_m, tiles_n;
     int out_f32, accumulate, group_m;

@@ -3,13 +3,14 @@
 //
 // The L2 -> LDS path, not the matrix cores, limits the smaller-tile kernels: bytes moved per
 // flop go with (1/BM + 1/BN).  A 256 x 256 tile moves two thirds of what 256 x 128 moves, but
-// one fp32 accumulator tile then fills all 256 AGPRs of a wave, so the Strassen / Winograd
-// recombination cannot keep its chains in registers.  Here exactly ONE accumulator lives in
-// registers and the chains are parked in private fp32 slabs (three per workgroup, 256 KiB
-// each, L2 resident, fully coalesced plain loads and stores -- no atomics):
-//   Winograd: 4 stores + 5 loads of a tile per tile job (the U-chain accumulates in place)
-//   Strassen: 9 stores + 9 loads
-// against 7 x 64 k-steps x 64 KiB of operand traffic.
+// one fp32 accumulator tile then fills all 256 AGPRs of a wave, so no Strassen / Winograd chain
+// can stay in registers beside it.  (Parking the chains in per-workgroup fp32 slabs was built
+// and measured: every CU parks 256 KiB at the same moment, nine to eighteen times per tile,
+// and the kernel ran a third slower than the 256 x 128 one.)  So this kernel only ever runs
+// plain products: one launch covers `nprod` independent products of equal shape (the seven
+// products of a level, each with its own operand pair and its own output matrix), product-major,
+// so that the chip works through one product at a time and each behaves like a classical GEMM.
+// The recombination of the seven outputs is a separate elementwise pass.
 //
 // Pipeline: k-steps of 64 (whole 128-byte lines per row), two LDS stages of 64 KiB, the
 // barrier of a step sits just before the next step's first fragments are read, at which
@@ -29,8 +30,6 @@ constexpr int kATile4 = kBM4 * kBK4 * 2;                 // 32 KiB
 constexpr int kBTile4 = kBN4 * kBK4 * 2;                 // 32 KiB
 constexpr int kStageBytes4 = kATile4 + kBTile4;          // 64 KiB
 constexpr int kSmemBytes4 = kStages4 * kStageBytes4;     // 128 KiB
-constexpr int kSlabFloats4 = kBM4 * kBN4;                // one parked tile
-constexpr int kSlabs4 = 3;
 
 // A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 64 w + 8 i + L/8, i = 0..7,
 // chunk (L%8) ^ ((row/2)%8).  n-contiguous B: 64 k-rows x 32 chunks (512 bytes); wave w loads
@@ -116,47 +115,7 @@ struct Acc4 {   // one 128 x 128 wave tile = 4 x 4 MFMA tiles = 256 registers
 #pragma unroll
                 for (int e = 0; e < 16; ++e) t[i][j][e] = 0.f;
     }
-    __device__ __forceinline__ void negate() {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) t[i][j] = -t[i][j];
-    }
 };
-
-// Parked tiles: lane-major groups of four registers, so every access is a contiguous KiB per wave.
-enum { PARK_SET = 0, PARK_ADD = 1 };
-__device__ __forceinline__ void park_store4(const Acc4& acc, float* slab) {
-    f32x4* p = reinterpret_cast<f32x4*>(slab) + threadIdx.x;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 v = {acc.t[i][j][4 * g], acc.t[i][j][4 * g + 1], acc.t[i][j][4 * g + 2], acc.t[i][j][4 * g + 3]};
-                p[((i * 4 + j) * 4 + g) * kThreads4] = v;
-                if (g == 3) __builtin_amdgcn_sched_barrier(0);   // one MFMA tile at a time: few temporaries
-            }
-}
-template <int MODE>
-__device__ __forceinline__ void park_load4(Acc4& acc, const float* slab) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(slab) + threadIdx.x;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const f32x4 v = p[((i * 4 + j) * 4 + g) * kThreads4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (MODE == PARK_SET) acc.t[i][j][4 * g + e] = v[e];
-                    else acc.t[i][j][4 * g + e] += v[e];
-                }
-                if (g == 3) __builtin_amdgcn_sched_barrier(0);
-            }
-}
 
 template <class T, bool B_KC>
 struct Pipe4 {
@@ -181,11 +140,19 @@ struct Pipe4 {
     __device__ __forceinline__ void start() {
         g = 0;
         slot = 0;
-        ld.issue(smem_addr);
-        if (!ld.done()) ld.issue(smem_addr + kStageBytes4);
-        if (total >= 2) wait_vmcnt_imm<16>(); else wait_vmcnt_imm<0>();   // step 0 has landed
+        if (STHIP_DBG & 4) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i] = u32x4{0, 0, 0, 0}; }
+        }
+        if (!(STHIP_DBG & 1)) {
+            ld.issue(smem_addr);
+            if (!ld.done()) ld.issue(smem_addr + kStageBytes4);
+            if (total >= 2) wait_vmcnt_imm<16>(); else wait_vmcnt_imm<0>();   // step 0 has landed
+        }
         __syncthreads();
-        read_frags(0, 0, 0);
+        if (!(STHIP_DBG & 4)) read_frags(0, 0, 0);
     }
 
     __device__ __forceinline__ void run(Acc4& acc, int KT) {
@@ -194,24 +161,27 @@ struct Pipe4 {
             for (int kg = 0; kg < 4; ++kg) {
                 const int nb = (kg + 1) & 1, cb = kg & 1;
                 if (kg < 3) {
-                    read_frags(nb, slot, kg + 1);
+                    if (!(STHIP_DBG & 4)) read_frags(nb, slot, kg + 1);
                 } else {
                     // Every wave has read all fragments of this step: after the barrier its stage is
                     // free for the step two ahead.  Step g+1 (the only load batch in flight) must
                     // have landed before its fragments are read.
-                    wait_vmcnt_imm<0>();
-                    __syncthreads();
-                    if (!ld.done()) ld.issue(smem_addr + slot * kStageBytes4);
-                    if (g + 1 < total) read_frags(nb, slot ^ 1, 0);
+                    if (!(STHIP_DBG & 1)) wait_vmcnt_imm<0>();
+                    if (!(STHIP_DBG & 2)) __syncthreads();
+                    if (!(STHIP_DBG & 1) && !ld.done()) ld.issue(smem_addr + slot * kStageBytes4);
+                    if (!(STHIP_DBG & 4) && g + 1 < total) read_frags(nb, slot ^ 1, 0);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
+                    for (int j = 0; j < 4; ++j)
+                        if (!(STHIP_DBG & 64)) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
+                if (!(STHIP_DBG & (4 | 64))) {
 #pragma unroll
-                for (int m = 0; m < 16; ++m) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+                    for (int m = 0; m < 16; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -264,18 +234,20 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
     }
 }
 
-template <class T, int ALGO, bool B_KC>
+template <class T, bool B_KC>
 __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    // blockIdx.x = product * tiles + tile: the XCD-aware renumbering works within one product
+    const int tiles = P.tiles_m * P.tiles_n;
+    const int prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
     GemmParams tp;
     tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = P.group_m;
     int tm, tn;
-    tile_coords(tp, tm, tn);
+    tile_coords_in(tp, (int)blockIdx.x - prod * tiles, tiles, tm, tn);
     const int tile_m = tm * kBM4, tile_n = tn * kBN4;
     const int batch = blockIdx.y;
-    char* Cb = reinterpret_cast<char*>(P.C) + (int64_t)batch * P.c_bs * (P.out_f32 ? 4 : 2);
+    char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    constexpr int NSEG = ALGO == ALGO_CLASSIC ? 1 : 7;
     const int KT = P.Kh / kBK4;
 
     Pipe4<T, B_KC> pipe;
@@ -283,90 +255,18 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     pipe.smem_addr = (uint32_t)(uintptr_t)(lptr_t)smem;
     pipe.wm = (wave >> 1) * 128;
     pipe.wn = (wave & 1) * 128;
-    pipe.total = NSEG * KT;
+    pipe.total = KT;
     pipe.ld.P = &P;
     pipe.ld.wave = wave;
-    pipe.ld.seg = 0; pipe.ld.kt = 0; pipe.ld.total_seg = NSEG; pipe.ld.KT = KT;
+    pipe.ld.seg = prod; pipe.ld.kt = 0; pipe.ld.total_seg = prod + 1; pipe.ld.KT = KT;
     pipe.ld.batch = batch; pipe.ld.tile_m = tile_m; pipe.ld.tile_n = tile_n;
     pipe.ld.point_at_segment();
     pipe.start();
 
-#define EMIT4(quad) store_tile4<T>(r, P, Cb, quad, tile_m + pipe.wm, tile_n + pipe.wn)
-    enum { Q11 = 0, Q12 = 1, Q21 = 2, Q22 = 3 };
     Acc4 r;
-    if constexpr (ALGO == ALGO_CLASSIC) {
-        r.zero();
-        pipe.run(r, KT);
-        EMIT4(Q11);
-    } else {
-        float* s0 = P.park + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (int64_t)(kSlabs4 * kSlabFloats4);
-        float* s1 = s0 + kSlabFloats4;
-        float* s2 = s1 + kSlabFloats4;
-        if constexpr (ALGO == ALGO_STRASSEN) {
-            // segment order M3 M6 M5 M7 M1 M2 M4
-            r.zero();
-            pipe.run(r, KT);                     // M3
-            park_store4(r, s0);                  // s0 = M3
-            pipe.run(r, KT);                     // + M6 -> C22 chain
-            park_store4(r, s1);                  // s1 = M3 + M6
-            r.zero();
-            pipe.run(r, KT);                     // M5
-            park_store4(r, s2);                  // s2 = M5
-            park_load4<PARK_ADD>(r, s0);
-            EMIT4(Q12);                          // C12 = M3 + M5
-            park_load4<PARK_SET>(r, s2);
-            r.negate();                          // C11 chain starts at -M5
-            pipe.run(r, KT);                     // + M7
-            park_store4(r, s0);                  // s0 = M7 - M5
-            r.zero();
-            pipe.run(r, KT);                     // M1
-            park_store4(r, s2);                  // s2 = M1
-            park_load4<PARK_ADD>(r, s1);
-            park_store4(r, s1);                  // s1 = M1 + M3 + M6
-            park_load4<PARK_SET>(r, s2);
-            park_load4<PARK_ADD>(r, s0);
-            park_store4(r, s0);                  // s0 = M1 - M5 + M7
-            r.zero();
-            pipe.run(r, KT);                     // M2
-            park_store4(r, s2);                  // s2 = M2
-            r.negate();
-            park_load4<PARK_ADD>(r, s1);
-            EMIT4(Q22);                          // C22 = M1 - M2 + M3 + M6
-            r.zero();
-            pipe.run(r, KT);                     // M4
-            park_store4(r, s1);                  // s1 = M4
-            park_load4<PARK_ADD>(r, s2);
-            EMIT4(Q21);                          // C21 = M2 + M4
-            park_load4<PARK_SET>(r, s1);
-            park_load4<PARK_ADD>(r, s0);
-            EMIT4(Q11);                          // C11 = M1 + M4 - M5 + M7
-        } else {
-            // segment order P1 P2 P6 P7 P5 P3 (-P4)
-            r.zero();
-            pipe.run(r, KT);                     // P1
-            park_store4(r, s0);                  // s0 = P1
-            pipe.run(r, KT);                     // + P2
-            EMIT4(Q11);                          // C11 = P1 + P2
-            park_load4<PARK_SET>(r, s0);
-            pipe.run(r, KT);                     // + P6 -> U2
-            park_store4(r, s0);                  // s0 = U2
-            pipe.run(r, KT);                     // + P7 -> U3
-            park_store4(r, s1);                  // s1 = U3
-            r.zero();
-            pipe.run(r, KT);                     // P5
-            park_store4(r, s2);                  // s2 = P5
-            park_load4<PARK_ADD>(r, s0);         // U4 = U2 + P5
-            pipe.run(r, KT);                     // + P3
-            EMIT4(Q12);                          // C12 = U4 + P3
-            park_load4<PARK_SET>(r, s2);
-            park_load4<PARK_ADD>(r, s1);
-            EMIT4(Q22);                          // C22 = U3 + P5
-            park_load4<PARK_SET>(r, s1);
-            pipe.run(r, KT);                     // + A22 (-T4)
-            EMIT4(Q21);                          // C21 = U3 - P4
-        }
-    }
-#undef EMIT4
+    r.zero();
+    pipe.run(r, KT);
+    store_tile4<T>(r, P, Cb, 0, tile_m + pipe.wm, tile_n + pipe.wn);
 }
 
 }  // namespace sthip

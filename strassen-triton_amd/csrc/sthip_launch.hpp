@@ -88,15 +88,14 @@ hipError_t launch_gemm3(const Gemm2Params& p, int batch, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// 256 x 256 kernel (16-bit operands, A contiguous along k): tables indexed [b_kc].
-#define STHIP_DECLARE_TABLE4(T, A) extern const LaunchTable3 kLaunch4_##T##_##A;
-STHIP_DECLARE_TABLE4(1, 0) STHIP_DECLARE_TABLE4(1, 1) STHIP_DECLARE_TABLE4(1, 2)
-STHIP_DECLARE_TABLE4(2, 0) STHIP_DECLARE_TABLE4(2, 1) STHIP_DECLARE_TABLE4(2, 2)
-#undef STHIP_DECLARE_TABLE4
+// 256 x 256 kernel (16-bit operands, A contiguous along k), p.nprod products per launch:
+// tables indexed [b_kc].
+extern const LaunchTable3 kLaunch4_1;
+extern const LaunchTable3 kLaunch4_2;
 
-template <class T, int ALGO, bool B_KC>
+template <class T, bool B_KC>
 hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
-    auto kern = gemm4_kernel<T, ALGO, B_KC>;
+    auto kern = gemm4_kernel<T, B_KC>;
     static bool opted[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -106,7 +105,8 @@ hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
         if (e != hipSuccess) return e;
         opted[dev] = true;
     }
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
+    const int nprod = p.nprod > 0 ? p.nprod : 1;
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, p);
     return hipGetLastError();
 }

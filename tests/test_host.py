@@ -46,7 +46,7 @@ def test_argument_errors_need_no_gpu():
     assert b"cannot be padded" in lib.sthip_last_error()
     # workspace.  One level: room for the ten quadrant sums (5 per operand) and the parked accumulator when the shape is
     # tile aligned, per batch entry; nothing for fp32, odd or unaligned shapes, or classic.
-    sums = lambda h: 2 * 5 * h * h * 2 + 3 * h * h * 4   # ten 16-bit sums + three parked fp32 tile sets
+    sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles)
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == sums(512)
     assert lib.sthip_workspace_bytes(3, 1024, 1024, 1024, 1, 1, 2, 1) == 3 * sums(512)
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == 0
