@@ -2,6 +2,7 @@
 // recursion for two or more Strassen levels, and the small element-wise kernels that
 // recursion needs.  See include/strassen_hip.h for the contract of every entry point.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -67,7 +68,7 @@ static const LaunchTable3* table4_for(int dt) {
     return dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
 }
 
-// STHIP_FORCE_TILE=128x128 | 256x128 | 256x256 overrides the tile table where the shape allows
+// STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 overrides the tile table where the shape allows
 // the forced tile (tuning and test aid); unset or anything else = automatic.
 static int forced_tile() {
     const char* e = getenv("STHIP_FORCE_TILE");
@@ -75,6 +76,7 @@ static int forced_tile() {
     if (!strcmp(e, "128x128")) return 2;
     if (!strcmp(e, "256x128")) return 3;
     if (!strcmp(e, "256x256")) return 4;
+    if (!strcmp(e, "128x128g")) return 5;   // 128 x 128 tiles, seven products as separate outputs
     return 0;
 }
 
@@ -94,7 +96,7 @@ struct ComboParams {
 };
 
 template <class T>
-__global__ void quad_combos_kernel(const ComboParams p) {
+__device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
     const int r = (int)(idx / p.chunks_per_row), c = (int)(idx % p.chunks_per_row);
@@ -133,6 +135,14 @@ __global__ void quad_combos_kernel(const ComboParams p) {
         *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.out[o]) + out_off) = w;
     }
 }
+
+template <class T>
+__global__ void __launch_bounds__(256) quad_combos_kernel(const ComboParams p) { quad_combos_body<T>(p); }
+
+// Both operands of a level in one launch: blockIdx.z picks the side.
+struct ComboPair { ComboParams side[2]; };
+template <class T>
+__global__ void __launch_bounds__(256) quad_combos_pair_kernel(const ComboPair pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
 
 // Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
 // Strassen (fixed_strassen.py:88-97): A side S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.
@@ -250,29 +260,31 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
         const int nout = algo == STHIP_STRASSEN ? 5 : 4;
-        for (int side = 0; side < 2 && (g_stages & 1); ++side) {
-            ComboParams cp;
-            memset(&cp, 0, sizeof(cp));
-            const bool kc = side == 0 ? a_kc : b_kc;
-            const int64_t r_ext = side == 0 ? (a_kc ? Mh : Kh) : (b_kc ? Nh : Kh);
-            const int64_t c_ext = side == 0 ? (a_kc ? Kh : Mh) : (b_kc ? Kh : Nh);
-            (void)kc;
-            for (int q = 0; q < 4; ++q) cp.q[q] = side == 0 ? Aq[q] : Bq[q];
-            for (int o = 0; o < nout; ++o) {
-                cp.out[o] = (side == 0 ? SA + (size_t)o * batch * sa_b : SB + (size_t)o * batch * sb_b);
-                for (int q = 0; q < 4; ++q)
-                    cp.coef[o][q] = algo == STHIP_STRASSEN ? (side == 0 ? kStrA[o][q] : kStrB[o][q])
-                                                           : (side == 0 ? kWinA[o][q] : kWinB[o][q]);
+        if (g_stages & 1) {
+            ComboPair pp;
+            memset(&pp, 0, sizeof(pp));
+            int64_t most = 0;
+            for (int side = 0; side < 2; ++side) {
+                ComboParams& cp = pp.side[side];
+                const int64_t r_ext = side == 0 ? (a_kc ? Mh : Kh) : (b_kc ? Nh : Kh);
+                const int64_t c_ext = side == 0 ? (a_kc ? Kh : Mh) : (b_kc ? Kh : Nh);
+                for (int q = 0; q < 4; ++q) cp.q[q] = side == 0 ? Aq[q] : Bq[q];
+                for (int o = 0; o < nout; ++o) {
+                    cp.out[o] = (side == 0 ? SA + (size_t)o * batch * sa_b : SB + (size_t)o * batch * sb_b);
+                    for (int q = 0; q < 4; ++q)
+                        cp.coef[o][q] = algo == STHIP_STRASSEN ? (side == 0 ? kStrA[o][q] : kStrB[o][q])
+                                                               : (side == 0 ? kWinA[o][q] : kWinB[o][q]);
+                }
+                cp.ld_in = side == 0 ? a_ld : b_ld;
+                cp.bs_in = side == 0 ? a_bs : b_bs;
+                cp.ld_out = side == 0 ? sa_ld : sb_ld;
+                cp.bs_out = (int64_t)((side == 0 ? sa_b : sb_b) / 2);
+                cp.nout = nout; cp.rows = (int)r_ext; cp.chunks_per_row = (int)(c_ext / 8);
+                most = std::max(most, r_ext * (c_ext / 8));
             }
-            cp.ld_in = side == 0 ? a_ld : b_ld;
-            cp.bs_in = side == 0 ? a_bs : b_bs;
-            cp.ld_out = side == 0 ? sa_ld : sb_ld;
-            cp.bs_out = (int64_t)((side == 0 ? sa_b : sb_b) / 2);
-            cp.nout = nout; cp.rows = (int)r_ext; cp.chunks_per_row = (int)(c_ext / 8);
-            const int64_t n = r_ext * (c_ext / 8);
-            dim3 grid((unsigned)ceil_div(n, 256), (unsigned)batch);
-            if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, stream, cp);
-            else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, stream, cp);
+            dim3 grid((unsigned)ceil_div(most, 256), (unsigned)batch, 2);
+            if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
+            else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
             int rc = check_launch("quad_combos");
             if (rc) return rc;
         }
@@ -317,26 +329,43 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     const LaunchTable3* t4 = table4_for(dt);
     const int force = forced_tile();
     const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
-    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && (!split || (!out_f32 && c_vec));
+    const bool grouped_ok = !split || (!out_f32 && c_vec);   // 16-bit products + recombination pass
+    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && grouped_ok;
     const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
+    const bool can5 = split && grouped_ok;
     const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch * (split ? 7 : 1);
     const int64_t tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
+    const int64_t tiles2 = (Mh / 128) * (Nh / 128) * batch;
+    // Measured on MI355X (bf16): the 256 x 256 grouped path wins from 4096^3 up when k is long
+    // enough to pay for writing the sums and the products (its extra passes cost bytes
+    // ~ MK + KN + MN, the products flops ~ MNK); when the 128 x 128 tiles of ONE product cannot
+    // fill the 256 CUs (small matrices, weight gradients with short M and N) the seven products
+    // side by side can, and that launch is 2 - 4 x faster; otherwise recombining in registers
+    // (no product round trip) is as fast or faster.
     int pick = 2;
-    if (can4 && tiles4 >= (split ? 400 : 224)) pick = 4;
+    if (can4 && tiles4 >= (split ? 400 : 224) && (!split || Kh >= 1024)) pick = 4;
+    else if (can5 && tiles2 < 256) pick = 5;
     else if (can3 && tiles3 >= 256) pick = 3;
     if (force == 4 && can4) pick = 4;
     else if (force == 3 && can3) pick = 3;
+    else if (force == 5 && can5) pick = 5;
     else if (force == 2) pick = 2;
-    if (pick == 4 && split) {
+    if ((pick == 4 || pick == 5) && split) {
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
         rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
         if (g_stages & 2) {
             p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
             p.out_f32 = 0; p.accumulate = 0; p.nprod = 7;
-            p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
-            p.group_m = 4;
-            e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+            if (pick == 4) {
+                p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
+                p.group_m = 4;
+                e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+            } else {
+                const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
+                if (!t) return 1;
+                e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+            }
             if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
         }
         if (g_stages & 4) {

@@ -48,8 +48,8 @@ struct Gemm2Params {
     void* C;
     float* park;          // scratch for one parked accumulator tile per workgroup (256 x 128 kernel, Strassen)
     int64_t c_rs, c_bs;   // C is row-major with unit column stride
-    int64_t c_ps;         // 256 x 256 kernel: element stride between the outputs of consecutive products
-    int nprod;            // 256 x 256 kernel: products in this launch (1 = plain GEMM)
+    int64_t c_ps;         // classical kernels: element stride between the outputs of consecutive products
+    int nprod;            // classical kernels: products in this launch (0 or 1 = plain GEMM)
     int Mh, Nh, Kh;       // extent of one segment product
     int tiles_m, tiles_n;
     int out_f32, accumulate, group_m;
@@ -238,10 +238,20 @@ __global__ void __launch_bounds__(kThreads) gemm2_kernel(const Gemm2Params P) {
     GemmParams tp;
     tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = P.group_m;
     int tm, tn;
-    tile_coords(tp, tm, tn);
+    // The classical kernel can run several independent products of equal shape in one launch
+    // (product-major: blockIdx.x = product * tiles + tile), each with its own operand pair
+    // (segment) and its own output matrix, c_ps elements apart.
+    int prod = 0;
+    if constexpr (ALGO == ALGO_CLASSIC) {
+        const int tiles = P.tiles_m * P.tiles_n;
+        prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
+        tile_coords_in(tp, (int)blockIdx.x - prod * tiles, tiles, tm, tn);
+    } else {
+        tile_coords(tp, tm, tn);
+    }
     const int tile_m = tm * 128, tile_n = tn * 128;
     const int batch = blockIdx.y;
-    char* Cb = reinterpret_cast<char*>(P.C) + (int64_t)batch * P.c_bs * (P.out_f32 ? 4 : 2);
+    char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int NSEG = ALGO == ALGO_CLASSIC ? 1 : 7;
     const int KT = P.Kh / kBK2;
@@ -254,7 +264,7 @@ __global__ void __launch_bounds__(kThreads) gemm2_kernel(const Gemm2Params P) {
     pipe.wn = (wave & 1) * 64;
     pipe.total = NSEG * KT;
     pipe.ld.P = &P;
-    pipe.ld.seg = 0; pipe.ld.kt = 0; pipe.ld.total_seg = NSEG; pipe.ld.KT = KT;
+    pipe.ld.seg = prod; pipe.ld.kt = 0; pipe.ld.total_seg = prod + NSEG; pipe.ld.KT = KT;
     pipe.ld.batch = batch; pipe.ld.tile_m = tile_m; pipe.ld.tile_n = tile_n;
     pipe.ld.point_at_segment();
     pipe.start();

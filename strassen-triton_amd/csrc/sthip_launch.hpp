@@ -59,7 +59,8 @@ hipError_t launch_gemm2(const Gemm2Params& p, int batch, hipStream_t stream) {
         if (e != hipSuccess) return e;
         opted[dev] = true;
     }
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
+    const int nprod = ALGO == ALGO_CLASSIC && p.nprod > 0 ? p.nprod : 1;
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads), kSmemBytes2, stream, p);
     return hipGetLastError();
 }

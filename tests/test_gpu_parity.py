@@ -230,7 +230,7 @@ def test_autograd_matmul(hip):
     assert torch.equal(A.grad, G @ B.detach().T) and torch.equal(B.grad, A.detach().T @ G)
 
 
-@pytest.mark.parametrize("tile", ["128x128", "256x128", "256x256"])
+@pytest.mark.parametrize("tile", ["128x128", "128x128g", "256x128", "256x256"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
 @pytest.mark.parametrize("tb", [False, True])
