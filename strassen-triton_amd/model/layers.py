@@ -5,8 +5,10 @@ the reference's model code are consumers of this layer, not part of it.
 """
 from __future__ import annotations
 
+import torch
 import torch.nn as nn
 
+import strassen_hip
 from fixed_strassen import LinearStrassen as _LinearStrassen
 from strassen import _strassen_base, strassen_matmul_two_layers
 
@@ -21,12 +23,67 @@ class LinearStrassen(_LinearStrassen):
         self.strassen_func = strassen_matmul_two_layers if depth == 2 else _strassen_base
 
 
-def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: int = 1):
+class _RectLinearFn(torch.autograd.Function):
+    """y = x W^T for any (rows, in) x (out, in): forward, dgrad dX = dY W and wgrad
+    dW = dY^T X are each one Strassen product over strided views, no padding, no copies."""
+
+    @staticmethod
+    def forward(ctx, x2d, weight, levels):
+        ctx.save_for_backward(x2d, weight)
+        ctx.levels = levels
+        return strassen_hip.gemm(x2d, weight.t(), levels=levels)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2d, weight = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = strassen_hip.gemm(dy, weight, levels=ctx.levels) if ctx.needs_input_grad[0] else None
+        dw = strassen_hip.gemm(dy.t(), x2d, levels=ctx.levels) if ctx.needs_input_grad[1] else None
+        return dx, dw, None
+
+
+class LinearStrassenRect(nn.Linear):
+    """nn.Linear of any shape whose three GEMMs are Strassen products.  Lifts the constraints
+    of the reference's layer (model/layers.py:240, :255-262: square, power of two, at most D
+    input rows, input padded to D x D): sizes that are odd or not tile multiples are handled
+    by the kernels' zero-padding edge tiles, so nothing is padded or sliced in memory."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=None,
+                 depth: int = 1, device: str = "cuda") -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        self.depth = depth
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        *batch_dims, d_in = input.shape
+        assert d_in == self.in_features, "Input dim mismatch"
+        x2d = input.reshape(-1, d_in)
+        y = _RectLinearFn.apply(x2d, self.weight, max(1, int(self.depth)))
+        if self.bias is not None:
+            y = y + self.bias
+        return y.view(*batch_dims, self.out_features)
+
+
+def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: int = 1,
+                                 square_only: bool = True):
     """Swap every square nn.Linear of at least min_size features for LinearStrassen, in
-    place, keeping weights and bias (reference model/layers.py:279-300)."""
+    place, keeping weights and bias (reference model/layers.py:279-300).  With
+    square_only=False, non-square layers (and squares that are not powers of two) whose smaller
+    side is at least min_size become LinearStrassenRect instead of being skipped; below
+    min_size a layer stays an nn.Linear, i.e. a classical GEMM."""
     for name, child in module.named_children():
-        if isinstance(child, nn.Linear) and not isinstance(child, _LinearStrassen):
-            if child.in_features == child.out_features and child.in_features >= min_size:
+        if isinstance(child, nn.Linear) and not isinstance(child, (_LinearStrassen, LinearStrassenRect)):
+            pow2 = child.in_features & (child.in_features - 1) == 0
+            if not square_only and min(child.in_features, child.out_features) >= min_size and \
+                    not (child.in_features == child.out_features and pow2):
+                print(f"Replacing '{name}' with LinearStrassenRect.")
+                new_layer = LinearStrassenRect(child.in_features, child.out_features,
+                                               bias=child.bias is not None, device=child.weight.device,
+                                               dtype=child.weight.dtype, depth=depth)
+                new_layer.weight.data.copy_(child.weight.data)
+                if child.bias is not None:
+                    new_layer.bias.data.copy_(child.bias.data)
+                setattr(module, name, new_layer)
+            elif child.in_features == child.out_features and child.in_features >= min_size:
                 print(f"Replacing '{name}' with LinearStrassen.")
                 new_layer = LinearStrassen(child.in_features, child.out_features,
                                            bias=child.bias is not None, device=child.weight.device,
@@ -38,4 +95,4 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
             else:
                 print(f"Skipping '{name}': Not square or too small.")
         elif len(list(child.children())) > 0:
-            replace_linear_with_strassen(child, min_size, depth)
+            replace_linear_with_strassen(child, min_size, depth, square_only)

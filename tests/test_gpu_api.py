@@ -117,6 +117,59 @@ def test_replace_linear_with_strassen(capsys):
     assert O.rel_fro(net(x).cpu(), before.cpu()) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(300, 768, 2304), (1000, 3072, 768), (77, 130, 129)])
+def test_linear_strassen_rect_forward_backward(dtype, shape):
+    """Non-square layer without padding: forward, dgrad and wgrad each against the same product
+    in fp64 (rel. Frobenius <= 1e-5 fp32 / 2e-2 bf16), and bit for bit on small integers."""
+    from model.layers import LinearStrassenRect
+    rows, d_in, d_out = shape
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    g = torch.Generator().manual_seed(7)
+    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda")
+    x = (torch.randn(rows, d_in, generator=g) * 0.5).to(dtype).cuda().requires_grad_()
+    dy = (torch.randn(rows, d_out, generator=g) * 0.5).to(dtype).cuda()
+    y = lin(x)
+    y.backward(dy)
+    W, b = lin.weight.detach().double(), lin.bias.detach().double()
+    rel = lambda got, ref: float(torch.linalg.norm(got.double() - ref) / torch.linalg.norm(ref))
+    assert y.shape == (rows, d_out)
+    assert rel(y.detach(), x.detach().double() @ W.T + b) <= tol
+    assert rel(x.grad, dy.double() @ W) <= tol
+    assert rel(lin.weight.grad, dy.double().T @ x.detach().double()) <= tol
+    assert rel(lin.bias.grad, dy.double().sum(0)) <= tol
+    # integers: every sum and product is exact, so the three GEMMs must be too
+    xi = torch.randint(-2, 3, (rows, d_in), generator=g).to(dtype).cuda().requires_grad_()
+    with torch.no_grad():
+        lin.weight.copy_(torch.randint(-1, 2, (d_out, d_in), generator=g).to(dtype))
+        lin.bias.zero_()
+    lin.weight.grad = None
+    di = torch.randint(-1, 2, (rows, d_out), generator=g).to(dtype).cuda()
+    yi = lin(xi.view(1, rows, d_in))
+    assert yi.shape == (1, rows, d_out)
+    yi.backward(di.view(1, rows, d_out))
+    Wi = lin.weight.detach().double()
+    exact = lambda got, ref: torch.equal(got.double(), ref.to(dtype).double())
+    assert exact(yi.detach()[0], xi.detach().double() @ Wi.T)
+    assert exact(xi.grad, di.double() @ Wi)
+    assert exact(lin.weight.grad, di.double().T @ xi.detach().double())
+
+
+def test_replace_linear_with_strassen_rect(capsys):
+    import torch.nn as nn
+    from model.layers import LinearStrassen, LinearStrassenRect, replace_linear_with_strassen
+    net = nn.Sequential(nn.Linear(256, 768), nn.GELU(), nn.Linear(768, 256), nn.Linear(256, 256),
+                        nn.Linear(256, 32)).cuda()
+    x = torch.randn(40, 256, device="cuda")
+    before = net(x)
+    replace_linear_with_strassen(net, min_size=128, depth=1, square_only=False)
+    out = capsys.readouterr().out
+    assert "Replacing '0' with LinearStrassenRect." in out and "Replacing '3' with LinearStrassen." in out
+    assert isinstance(net[0], LinearStrassenRect) and isinstance(net[2], LinearStrassenRect)
+    assert isinstance(net[3], LinearStrassen) and type(net[4]) is nn.Linear
+    assert O.rel_fro(net(x).cpu(), before.cpu()) <= 1e-5
+
+
 def test_cpu_tensors_are_refused():
     import fixed_strassen
     with pytest.raises(RuntimeError, match="no CPU implementation"):
