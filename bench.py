@@ -183,13 +183,13 @@ def main():
     kernel_s, prepass_s, recombine_s = ev / args.steps, 0.0, 0.0
     staged = levels == 1 and algo != "classic" and nbytes > 0
     if staged:
-        lib.sthip_debug_set_stages(2)
+        all_stages = lib.sthip_debug_set_stages(2)
         _, ev_k = time_gpu(fn, args.steps, 3)
         lib.sthip_debug_set_stages(1)
         _, ev_p = time_gpu(fn, args.steps, 3)
         lib.sthip_debug_set_stages(4)
         _, ev_r = time_gpu(fn, args.steps, 3)
-        lib.sthip_debug_set_stages(7)
+        lib.sthip_debug_set_stages(all_stages)
         kernel_s, prepass_s, recombine_s = ev_k / args.steps, ev_p / args.steps, ev_r / args.steps
         fn()   # leave `out` holding a complete result for the error figures below
 

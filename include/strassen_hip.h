@@ -57,7 +57,10 @@ enum sthip_algo {
  * runs the seven products.  Large problems (half-size blocks multiples of 256, result in the
  * operand type) use 256 x 256 tiles, round each product once to the operand type as the
  * reference's mm does, and recombine in a third pass in fp32; the others recombine in
- * registers without that rounding.  levels >= 2 recurses on
+ * registers without that rounding.  levels = 2 on tile-aligned 16-bit problems runs as five
+ * launches (sums of both levels, ONE grouped GEMM of the 49 quarter-size products, two
+ * recombination passes; every level returns its products in the operand type, the first level
+ * is always Strassen).  Otherwise levels >= 2 recurses on
  * the host (sums and products of the upper levels in workspace) and requires the workspace.
  *
  * Replaces: _strassen_base (fixed_strassen.py:11-57, fixed_strassen_fp32_agg.py:12-56),
@@ -118,7 +121,8 @@ int sthip_debug_transpose_read(void* out, void* stream);
 
 /* Profiling aid: selects which stages of the pipelined one-level path later calls run
  * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM, bit 2 = recombination pass of the
- * 256 x 256 path; default 7) and returns the previous mask.  With mask 2 the GEMM re-uses the
+ * grouped paths; bit 3 lets two-level calls run as one 49-product launch instead of the host
+ * recursion; default 15) and returns the previous mask.  With mask 2 the GEMM re-uses the
  * sums a previous call left in the same workspace, so the dominant kernel can be timed alone.
  * Process-wide; not for production calls.  No counterpart in the reference. */
 int sthip_debug_set_stages(int mask);

@@ -16,7 +16,7 @@ namespace sthip {
 static thread_local char g_err[512] = "";
 // Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM.
 // Only the profiling hook sthip_debug_set_stages changes it.
-static int g_stages = 7;
+static int g_stages = 15;
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -144,6 +144,11 @@ struct ComboPair { ComboParams side[2]; };
 template <class T>
 __global__ void __launch_bounds__(256) quad_combos_pair_kernel(const ComboPair pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
 
+// The fourteen operands of the seven products of a level (second-level sums) in one launch.
+struct ComboMany { ComboParams side[14]; };
+template <class T>
+__global__ void __launch_bounds__(256) quad_combos_many_kernel(const ComboMany pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
+
 // Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
 // Strassen (fixed_strassen.py:88-97): A side S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.
 static const signed char kStrA[5][4] = {{1, 1, 0, 0}, {0, 0, 1, 1}, {1, 0, 0, 1}, {0, 1, 0, -1}, {-1, 0, 1, 0}};
@@ -165,10 +170,12 @@ static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
 // add in fp32 in the reference's order (fixed_strassen_fp32_agg.py:44-53), round once.  One
 // thread per 16-byte chunk of a half-size row.
 struct Recombine16Params {
-    const void* prod;     // [batch][7][Mh x Nh]
+    const void* prod;     // [batch][7] dense Mh x Nh matrices, p_ps elements apart
     void* C;
     int64_t c_rs, c_bs;   // elements
+    int64_t p_ps;
     int Mh, Nh, accumulate;
+    int out_f32;          // C is fp32 (no final rounding) instead of the operand type
 };
 
 template <class T>
@@ -186,7 +193,7 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.Mh * nq) return;
     const int i = (int)(idx / nq), j = (int)(idx % nq) * 8;
-    const int64_t blk = (int64_t)p.Mh * p.Nh;
+    const int64_t blk = p.p_ps;
     const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)blockIdx.y * 7 * blk + (int64_t)i * p.Nh + j) * 2;
     float m[7][8];
 #pragma unroll
@@ -206,6 +213,17 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
             out[2][e] = u3 + m[6][e];                                // C21 = U3 - P4
             out[3][e] = u3 + m[4][e];                                // C22 = U3 + P5
         }
+    }
+    if (p.out_f32) {
+        float* Cf = reinterpret_cast<float*>(p.C) + (int64_t)blockIdx.y * p.c_bs;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            f32x4* d = reinterpret_cast<f32x4*>(Cf + (int64_t)(i + (q >> 1) * p.Mh) * p.c_rs + (j + (q & 1) * p.Nh));
+            f32x4 lo = {out[q][0], out[q][1], out[q][2], out[q][3]}, hi = {out[q][4], out[q][5], out[q][6], out[q][7]};
+            if (p.accumulate) { lo += d[0]; hi += d[1]; }
+            d[0] = lo; d[1] = hi;
+        }
+        return;
     }
     char* Cb = reinterpret_cast<char*>(p.C) + (int64_t)blockIdx.y * p.c_bs * 2;
 #pragma unroll
@@ -353,7 +371,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     if ((pick == 4 || pick == 5) && split) {
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
-        rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
+        rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0; rp.p_ps = Mh * Nh; rp.out_f32 = 0;
         if (g_stages & 2) {
             p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
             p.out_f32 = 0; p.accumulate = 0; p.nprod = 7;
@@ -557,9 +575,8 @@ static bool combos_ok(View X, int64_t r_blk, int64_t c_blk) {
     return false;
 }
 
-static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, size_t out_stride, int nout,
-                      const signed char (*coef)[4], hipStream_t stream) {
-    ComboParams cp;
+static int64_t fill_combo(ComboParams& cp, View X, int64_t r_blk, int64_t c_blk, char* out, size_t out_stride,
+                          int nout, const signed char (*coef)[4]) {
     memset(&cp, 0, sizeof(cp));
     const bool row_major = X.cs == 1;
     for (int q = 0; q < 4; ++q)
@@ -572,12 +589,157 @@ static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, s
     cp.ld_in = row_major ? X.rs : X.cs;
     cp.ld_out = cols;
     cp.nout = nout; cp.rows = (int)rows; cp.chunks_per_row = (int)(cols / 8);
-    const int64_t n = rows * (cols / 8);
+    return rows * (cols / 8);
+}
+
+static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, size_t out_stride, int nout,
+                      const signed char (*coef)[4], hipStream_t stream) {
+    ComboParams cp;
+    const int64_t n = fill_combo(cp, X, r_blk, c_blk, out, out_stride, nout, coef);
     if (n == 0) return STHIP_OK;
     dim3 grid((unsigned)ceil_div(n, 256), 1);
     if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, stream, cp);
     else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, stream, cp);
     return check_launch("quad_combos");
+}
+
+// Operand pairs of the seven products of one level, in kernel order (Strassen M3 M6 M5 M7 M1 M2 M4,
+// Winograd P1 P2 P6 P7 P5 P3 -P4).  X is mh x kh blocks of A, Y is kh x nh blocks of B; a raw
+// quadrant is a view into the operand, a sum is dense in the operand's storage orientation at
+// S? + index * stride (index = output number of kStr? / kWin?).
+static void level_operands(int algo, View A, View B, int64_t mh, int64_t nh, int64_t kh,
+                           const char* SA, size_t sa_b, const char* SB, size_t sb_b, View xa[7], View xb[7]) {
+    auto rawA = [&](int q) { return View{A.p + ((int64_t)(q >> 1) * mh * A.rs + (int64_t)(q & 1) * kh * A.cs) * 2, A.rs, A.cs}; };
+    auto rawB = [&](int q) { return View{B.p + ((int64_t)(q >> 1) * kh * B.rs + (int64_t)(q & 1) * nh * B.cs) * 2, B.rs, B.cs}; };
+    auto sumA = [&](int o) { const char* p = SA + (size_t)o * sa_b; return A.cs == 1 ? View{p, kh, 1} : View{p, 1, mh}; };
+    auto sumB = [&](int o) { const char* p = SB + (size_t)o * sb_b; return B.cs == 1 ? View{p, nh, 1} : View{p, 1, kh}; };
+    if (algo == STHIP_STRASSEN) {
+        xa[0] = rawA(0); xb[0] = sumB(0);   // M3 = A11 S1
+        xa[1] = sumA(4); xb[1] = sumB(4);   // M6 = S9 S10
+        xa[2] = sumA(0); xb[2] = rawB(3);   // M5 = S2 B22
+        xa[3] = sumA(3); xb[3] = sumB(3);   // M7 = S7 S8
+        xa[4] = sumA(2); xb[4] = sumB(2);   // M1 = S5 S6
+        xa[5] = sumA(1); xb[5] = rawB(0);   // M2 = S3 B11
+        xa[6] = rawA(3); xb[6] = sumB(1);   // M4 = A22 S4
+    } else {
+        xa[0] = rawA(0); xb[0] = rawB(0);   // P1 = A11 B11
+        xa[1] = rawA(1); xb[1] = rawB(2);   // P2 = A12 B21
+        xa[2] = sumA(1); xb[2] = sumB(1);   // P6 = S2 T2
+        xa[3] = sumA(2); xb[3] = sumB(2);   // P7 = S3 T3
+        xa[4] = sumA(0); xb[4] = sumB(0);   // P5 = S1 T1
+        xa[5] = sumA(3); xb[5] = rawB(3);   // P3 = S4 B22
+        xa[6] = rawA(3); xb[6] = sumB(3);   // -P4 = A22 (-T4)
+    }
+}
+
+static int launch_recombine16(int dt, int algo, const void* prod, int64_t p_ps, char* C, int64_t c_rs, int64_t c_bs,
+                              int64_t batch, int64_t Mh, int64_t Nh, bool accumulate, bool out_f32, hipStream_t stream) {
+    Recombine16Params rp;
+    rp.out_f32 = out_f32 ? 1 : 0;
+    rp.prod = prod; rp.p_ps = p_ps; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
+    rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
+    dim3 grid((unsigned)ceil_div(Mh * (Nh / 8), 256), (unsigned)batch);
+#define GO(T, A) hipLaunchKernelGGL((recombine16_kernel<T, A>), grid, dim3(256), 0, stream, rp)
+    if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
+    else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
+#undef GO
+    return check_launch("recombine16");
+}
+
+// Two levels as five launches: sums of the first level, sums of the second level for all seven
+// first-level products at once, ONE grouped GEMM of the 49 quarter-size products (the schedule
+// the reference's two-layer Triton kernel runs per tile, strassen.py:373-611, here on whole
+// matrices), recombination of the 49 into the seven first-level products, recombination of
+// those into C.  Every level returns its result in the operand type, as the reference's
+// recursion does (fixed_strassen_fp32_agg.py:47-50); the first level is always Strassen.
+// Needs: 16-bit operands, whole aligned problem, C in the operand type with 16-byte aligned rows.
+static size_t two_level_bytes(int64_t mh, int64_t nh, int64_t kh) {
+    const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
+    return 5 * (align256(mh * kh * 2) + align256(kh * nh * 2)) + 35 * (align256(mq * kq * 2) + align256(kq * nq * 2)) +
+           49 * align256(mq * nq * 2) + 7 * align256(mh * nh * 2);
+}
+
+static bool two_level_shape(int dt, int64_t mh, int64_t nh, int64_t kh) {
+    return mh % 2 == 0 && nh % 2 == 0 && kh % 2 == 0 && fast_shape(dt, mh / 2, nh / 2, kh / 2);
+}
+
+static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int64_t nh, int64_t kh,
+                          int dt, int algo, bool accumulate, bool out_f32, char* ws, hipStream_t stream) {
+    const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
+    const size_t sa1 = align256(mh * kh * 2), sb1 = align256(kh * nh * 2);
+    const size_t sa2 = align256(mq * kq * 2), sb2 = align256(kq * nq * 2);
+    const size_t pb = align256(mq * nq * 2), mb = align256(mh * nh * 2);
+    char* SA1 = ws;
+    char* SB1 = SA1 + 5 * sa1;
+    char* SA2 = SB1 + 5 * sb1;
+    char* SB2 = SA2 + 35 * sa2;
+    char* P = SB2 + 35 * sb2;
+    char* Mp = P + 49 * pb;
+    const bool a_kc = A.cs == 1, b_kc = B.rs == 1;
+    const int nout2 = algo == STHIP_STRASSEN ? 5 : 4;
+
+    // first-level sums (Strassen)
+    {
+        ComboPair pp;
+        const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA);
+        const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
+        else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos (level 1)");
+        if (rc) return rc;
+    }
+    View xa1[7], xb1[7];
+    level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1);
+
+    // second-level sums of all fourteen operands
+    {
+        ComboMany pm;
+        int64_t most = 0;
+        for (int p = 0; p < 7; ++p) {
+            most = std::max(most, fill_combo(pm.side[2 * p], xa1[p], mq, kq, SA2 + (size_t)p * 5 * sa2, sa2, nout2,
+                                             algo == STHIP_STRASSEN ? kStrA : kWinA));
+            most = std::max(most, fill_combo(pm.side[2 * p + 1], xb1[p], kq, nq, SB2 + (size_t)p * 5 * sb2, sb2, nout2,
+                                             algo == STHIP_STRASSEN ? kStrB : kWinB));
+        }
+        dim3 grid((unsigned)ceil_div(most, 256), 1, 14);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_many_kernel<bf16_t>, grid, dim3(256), 0, stream, pm);
+        else hipLaunchKernelGGL(quad_combos_many_kernel<f16_t>, grid, dim3(256), 0, stream, pm);
+        int rc = check_launch("quad_combos (level 2)");
+        if (rc) return rc;
+    }
+
+    // the 49 products, product-major: first-level product p, second-level product j -> P[7 p + j]
+    Gemm2Params g;
+    memset(&g, 0, sizeof(g));
+    for (int p = 0; p < 7; ++p) {
+        View xa2[7], xb2[7];
+        level_operands(algo, xa1[p], xb1[p], mq, nq, kq, SA2 + (size_t)p * 5 * sa2, sa2, SB2 + (size_t)p * 5 * sb2, sb2, xa2, xb2);
+        for (int j = 0; j < 7; ++j)
+            g.seg[7 * p + j] = Seg2{xa2[j].p, xb2[j].p, a_kc ? xa2[j].rs : xa2[j].cs, b_kc ? xb2[j].cs : xb2[j].rs, 0, 0};
+    }
+    g.C = P; g.c_rs = nq; g.c_ps = (int64_t)(pb / 2); g.c_bs = 0;
+    g.Mh = (int)mq; g.Nh = (int)nq; g.Kh = (int)kq;
+    g.out_f32 = 0; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
+    const LaunchTable3* t4 = table4_for(dt);
+    const bool big = a_kc && t4 && mq % kBM4 == 0 && nq % kBN4 == 0 && kq >= 1024 && forced_tile() != 5 && forced_tile() != 2;
+    hipError_t e;
+    if (big) {
+        g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
+        e = t4->fn[b_kc ? 1 : 0](g, 1, stream);
+    } else {
+        const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
+        if (!t) return fail(STHIP_ERR_DTYPE, "no 16-bit kernel for dtype %d", dt);
+        g.tiles_m = (int)(mq / 128); g.tiles_n = (int)(nq / 128);
+        g.group_m = 8;
+        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](g, 1, stream);
+    }
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+
+    // 49 -> 7 (second-level recombination, one batch entry per first-level product), then 7 -> C
+    int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
+    if (rc) return rc;
+    return launch_recombine16(dt, STHIP_STRASSEN, Mp, (int64_t)(mb / 2), C, c_rs, 0, 1, mh, nh, accumulate, out_f32, stream);
 }
 
 // Vector form of recombine_kernel: four consecutive columns per thread (nh % 4 == 0, C with unit
@@ -659,8 +821,12 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
     if (levels <= 0) return 0;
     if (levels == 1) return fast_shape(dt, mh, nh, kh) ? prepass_bytes(1, mh, nh, kh) : 0;
     const size_t es = elem_size(dt);
-    return 5 * (align256(mh * kh * es) + align256(kh * nh * es)) + 7 * align256(mh * nh * 4) +
-           workspace_for(mh, nh, kh, dt, levels - 1);
+    const size_t recursive = 5 * (align256(mh * kh * es) + align256(kh * nh * es)) + 7 * align256(mh * nh * 4) +
+                             workspace_for(mh, nh, kh, dt, levels - 1);
+    // two levels may run as one 49-product launch (two_level_flat) or, if the call's layout or
+    // result type rules that out, as the host recursion: room for either
+    if (levels == 2 && two_level_shape(dt, mh, nh, kh)) return std::max(recursive, two_level_bytes(mh, nh, kh));
+    return recursive;
 }
 
 // C (+)= A x B with `levels` levels.  (Mp, Np, Kp) >= (M, N, K) are the padded sizes the
@@ -668,7 +834,9 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
 static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                     int64_t M, int64_t N, int64_t K, int64_t Mp, int64_t Np, int64_t Kp,
                     int dt, int out_dt, int algo, int levels, bool accumulate,
-                    char* ws, size_t ws_bytes, hipStream_t stream) {
+                    char* ws, size_t ws_bytes, hipStream_t stream, bool inner = false) {
+    // inner: this product is one of the seven of an upper level, which wants it in fp32; it may
+    // still be formed from 16-bit sub-products (only the last rounding is skipped).
     const bool out_f32 = out_dt == STHIP_F32;
     if (algo == STHIP_CLASSIC || levels <= 0)
         return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, 0, 0, 0, dt, out_f32, STHIP_CLASSIC, accumulate,
@@ -679,7 +847,19 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                             ws, ws_bytes, stream);
 
     const size_t es = elem_size(dt);
-    const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es), m_b = align256(mh * nh * 4);
+    if (levels == 2 && (g_stages & 8) && two_level_shape(dt, mh, nh, kh) && (!out_f32 || inner) && M == Mp && N == Np && K == Kp &&
+        c_cs == 1 && c_rs % 8 == 0 && aligned_to(C, 16) && combos_ok(A, mh, kh) && combos_ok(B, kh, nh) &&
+        (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1)) {
+        const size_t flat = two_level_bytes(mh, nh, kh);
+        if (!ws || !aligned_to(ws, 256) || ws_bytes < flat)
+            return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, flat);
+        return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, stream);
+    }
+    // Whole, aligned 16-bit problems: all five sums of each operand in one bandwidth-bound launch.
+    const bool whole = M == Mp && N == Np && K == Kp;
+    const bool vec = dt != STHIP_F32 && whole && combos_ok(A, mh, kh) && combos_ok(B, kh, nh);
+    const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es);
+    const size_t m_b = align256(mh * nh * 4);
     const size_t need = 5 * (sa_b + sb_b) + 7 * m_b;
     if (!ws || ws_bytes < need) return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, need);
     char* SA = ws;
@@ -688,9 +868,6 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     char* child_ws = ws + need;
     const size_t child_bytes = ws_bytes - need;
 
-    // Whole, aligned 16-bit problems: all five sums of each operand in one bandwidth-bound launch.
-    const bool whole = M == Mp && N == Np && K == Kp;
-    const bool vec = dt != STHIP_F32 && whole && combos_ok(A, mh, kh) && combos_ok(B, kh, nh);
     if (vec) {
         int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, stream);
         if (rc) return rc;
@@ -728,7 +905,7 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             b = {SB, nh, 1};
         }
         int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, mh, nh, kh, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
-                          false, child_ws, child_bytes, stream);
+                          false, child_ws, child_bytes, stream, true);
         if (rc) return rc;
     }
     return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, stream);
@@ -843,7 +1020,7 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
 
 int sthip_debug_set_stages(int mask) {
     const int old = g_stages;
-    g_stages = mask & 7;
+    g_stages = mask & 15;
     return old;
 }
 

@@ -30,7 +30,7 @@ namespace sthip {
 #define STHIP_DBG 0
 #endif
 
-constexpr int kMaxSeg = 7;
+constexpr int kMaxSeg = 49;   // seven products of one level, or the 49 of two levels in one launch
 constexpr int kStages = 4;
 constexpr int kBK2 = 64;                       // k per step (16-bit operands)
 constexpr int kTileBytes2 = 128 * kBK2 * 2;    // one operand tile: 16 KiB

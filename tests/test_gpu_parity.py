@@ -222,6 +222,62 @@ def test_config5_gpt2_linears(hip, d_in, d_out):
         assert e_ref <= TOL[torch.bfloat16] and e_exact <= TOL[torch.bfloat16], (name, e_ref, e_exact)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("algo", ["strassen", "winograd"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("shape", [(512, 512, 256), (1024, 512, 512), (2048, 2048, 4096)])
+def test_two_levels_as_one_launch(hip, dtype, algo, ta, tb, shape):
+    """Tile-aligned 16-bit two-level calls run as ONE grouped launch of the 49 quarter-size
+    products (256 x 256 tiles for the largest shape, 128 x 128 for the others).  Entries in
+    [-1, 1] and short k keep every sum and every 16-bit product an exactly representable
+    integer, so the result must equal the classical product bit for bit; on random inputs it
+    must agree with the host recursion (stage bit 3 off) and with fp64 inside the tolerance."""
+    from strassen_hip import _capi
+    M, N, K = shape
+    if K <= 512:
+        A, B = _ints((M, K), 41, -1, 1, dtype), _ints((K, N), 42, -1, 1, dtype)
+        C = hip.gemm(_layout(A, ta), _layout(B, tb), algo=algo, levels=2)
+        exact = A.double() @ B.double()
+        assert float(exact.abs().max()) <= 256
+        assert torch.equal(C.cpu().double(), exact)
+        C0 = _ints((M, N), 43, -3, 3, dtype).cuda()
+        Cacc = C0.clone()
+        hip.gemm(_layout(A, ta), _layout(B, tb), out=Cacc, algo=algo, levels=2, accumulate=True)
+        want = (C0.cpu().double() + exact).to(dtype)
+        assert torch.equal(Cacc.cpu(), want)
+    A = _gauss((M, K), 44, K ** -0.5, dtype)
+    B = _gauss((K, N), 45, 1.0, dtype)
+    Ag, Bg = _layout(A, ta), _layout(B, tb)
+    flat = hip.gemm(Ag, Bg, algo=algo, levels=2)
+    lib = _capi.load()
+    prev = lib.sthip_debug_set_stages(7)
+    try:
+        rec = hip.gemm(Ag, Bg, algo=algo, levels=2)
+    finally:
+        lib.sthip_debug_set_stages(prev)
+    ref = Ag.double() @ Bg.double()
+    rel = lambda X: float(torch.linalg.norm(X.double() - ref) / torch.linalg.norm(ref))
+    assert rel(flat) <= TOL[dtype] and rel(rec) <= TOL[dtype]
+    assert float(torch.linalg.norm(flat.double() - rec.double()) / torch.linalg.norm(ref)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tb", [False, True])
+def test_three_levels_16bit(hip, dtype, tb):
+    """Three levels on an aligned 16-bit problem: the top level keeps its seven products in the
+    operand type and hands each to the 49-product launch.  Exact on entries in [-1, 1] with
+    short k; random inputs inside the tolerance of fp64."""
+    A, B = _ints((1024, 512), 51, -1, 1, dtype), _ints((512, 1024), 52, -1, 1, dtype)
+    C = hip.gemm(A.cuda(), _layout(B, tb), algo="strassen", levels=3)
+    exact = A.double() @ B.double()
+    assert float(exact.abs().max()) <= 256 and torch.equal(C.cpu().double(), exact)
+    A, B = _gauss((2048, 1024), 53, 1024 ** -0.5, dtype), _gauss((1024, 2048), 54, 1.0, dtype)
+    Ag, Bg = A.cuda(), _layout(B, tb)
+    C = hip.gemm(Ag, Bg, algo="strassen", levels=3)
+    ref = Ag.double() @ Bg.double()
+    assert float(torch.linalg.norm(C.double() - ref) / torch.linalg.norm(ref)) <= TOL[dtype]
+
+
 def test_autograd_matmul(hip):
     A = _ints((256, 128), 31, -1, 1).cuda().requires_grad_()
     B = _ints((128, 384), 32, -1, 1).cuda().requires_grad_()

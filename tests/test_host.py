@@ -52,12 +52,18 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
-    # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace.
+    # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace
+    # (host recursion), or -- for tile-aligned 16-bit problems, which may run as one 49-product launch --
+    # ten half-size sums, 70 quarter-size sums, 49 quarter-size products and seven half-size products;
+    # the query covers whichever is larger.
     upper = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
+    flat = lambda h: 10 * h * h * 2 + (70 + 49) * (h // 2) ** 2 * 2 + 7 * h * h * 2
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
-    assert two == upper(512) + sums(256)
+    assert two == max(upper(512) + sums(256), flat(512))
     three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
-    assert three == upper(512) + upper(256) + sums(128)
+    assert three == upper(512) + max(upper(256) + sums(128), flat(256))
+    # fp32 never takes the one-launch form
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4
 
 
 def test_reference_recursion_depth():
