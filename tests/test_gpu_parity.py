@@ -281,6 +281,29 @@ def test_three_levels_16bit(hip, dtype, tb):
     assert float(torch.linalg.norm(C.double() - ref) / torch.linalg.norm(ref)) <= 2 * TOL[dtype]
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 320), (1024, 1024, 1024)])
+def test_fp32_batched_products(hip, monkeypatch, ta, tb, shape):
+    """fp32, one level, tile-aligned: the seven products run as one batched classical launch
+    over dense operand copies.  Exact on integers; on random inputs within 1e-5 of fp64 and of
+    the fused kernel (forced with STHIP_FORCE_TILE=128x128), also when accumulating into C."""
+    M, N, K = shape
+    A, B = _ints((M, K), 61), _ints((K, N), 62)
+    Ag, Bg = _layout(A, ta), _layout(B, tb)
+    assert torch.equal(hip.gemm(Ag, Bg, algo="strassen", levels=1).cpu().double(), A.double() @ B.double())
+    A, B = _gauss((M, K), 63, K ** -0.5, torch.float32), _gauss((K, N), 64, 1.0, torch.float32)
+    Ag, Bg = _layout(A, ta), _layout(B, tb)
+    C0 = _gauss((M, N), 65, 1.0, torch.float32).cuda()
+    got = hip.gemm(Ag, Bg, algo="strassen", levels=1)
+    acc = hip.gemm(Ag, Bg, out=C0.clone(), algo="strassen", levels=1, accumulate=True)
+    monkeypatch.setenv("STHIP_FORCE_TILE", "128x128")
+    fused = hip.gemm(Ag, Bg, algo="strassen", levels=1)
+    ref = Ag.double() @ Bg.double()
+    rel = lambda X, R: float(torch.linalg.norm(X.double() - R) / torch.linalg.norm(R))
+    assert rel(got, ref) <= 1e-5 and rel(fused, ref) <= 1e-5 and rel(got, fused.double()) <= 1e-5
+    assert rel(acc, ref + C0.double()) <= 1e-5
+
+
 def test_autograd_matmul(hip):
     A = _ints((256, 128), 31, -1, 1).cuda().requires_grad_()
     B = _ints((128, 384), 32, -1, 1).cuda().requires_grad_()

@@ -49,7 +49,10 @@ def test_argument_errors_need_no_gpu():
     sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles)
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == sums(512)
     assert lib.sthip_workspace_bytes(3, 1024, 1024, 1024, 1, 1, 2, 1) == 3 * sums(512)
-    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == 0
+    # fp32, tile aligned: seven dense A operands, seven B operands, seven fp32 products
+    f32 = lambda h: 7 * 3 * h * h * 4
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == f32(512)
+    assert lib.sthip_workspace_bytes(1, 1000, 1000, 1000, 0, 0, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
     # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace
@@ -63,7 +66,7 @@ def test_argument_errors_need_no_gpu():
     three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
     assert three == upper(512) + max(upper(256) + sums(128), flat(256))
     # fp32 never takes the one-launch form
-    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4 + f32(256)
 
 
 def test_reference_recursion_depth():
