@@ -104,7 +104,8 @@ __device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
     const int64_t out_off = ((int64_t)blockIdx.y * p.bs_out + (int64_t)r * p.ld_out + c * 8) * 2;
     u32x4 v[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.q[q]) + in_off);
+    for (int q = 0; q < 4; ++q)
+        v[q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.q[q]) + in_off));
     float x[4][8];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -223,7 +224,7 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
     const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)blockIdx.y * 7 * blk + (int64_t)i * p.Nh + j) * 2;
     float m[7][8];
 #pragma unroll
-    for (int q = 0; q < 7; ++q) unpack8<T>(*reinterpret_cast<const u32x4*>(src + q * blk * 2), m[q]);
+    for (int q = 0; q < 7; ++q) unpack8<T>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + q * blk * 2)), m[q]);
     float out[4][8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -267,7 +268,7 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
             if constexpr (__is_same(T, bf16_t)) w[k] = pack_bf16(out[q][2 * k], out[q][2 * k + 1]);
             else w[k] = pack_f16(out[q][2 * k], out[q][2 * k + 1]);
         }
-        *d = w;
+        __builtin_nontemporal_store(w, d);
     }
 }
 
