@@ -10,10 +10,12 @@ stream, and the grid is limited by --max-n.
 
     python main_profiling.py [--dtype bf16|fp16|fp32] [--max-n 16384] [--min-n 1024]
     python main_profiling.py --gpt2      # the Linear shapes of GPT-2 small, forward and backward
+    python main_profiling.py --json out.json   # also write the rows as JSON
 """
 from __future__ import annotations
 
 import argparse
+import json
 
 import torch
 import torch.nn as nn
@@ -154,11 +156,15 @@ if __name__ == "__main__":
     ap.add_argument("--min-n", type=int, default=1024)
     ap.add_argument("--max-n", type=int, default=16384)
     ap.add_argument("--gpt2", action="store_true", help="GPT-2-small Linear shapes instead of the square grid")
+    ap.add_argument("--json", default=None, help="write the measured rows to this file as JSON")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: this benchmark needs an MI355X")
     print(f"device: {torch.cuda.get_device_name(0)}  dtype: {args.dtype}")
     if args.gpt2:
-        profile_gpt2_linears(dtype=_DTYPES[args.dtype])
+        rows = profile_gpt2_linears(dtype=_DTYPES[args.dtype])
     else:
-        profile_linear_layers(_DTYPES[args.dtype], args.min_n, args.max_n)
+        rows = profile_linear_layers(_DTYPES[args.dtype], args.min_n, args.max_n)
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump({"device": torch.cuda.get_device_name(0), "dtype": args.dtype, "rows": rows}, f, indent=1)

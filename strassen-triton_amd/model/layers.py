@@ -67,14 +67,12 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
                                  square_only: bool = True):
     """Swap every square nn.Linear of at least min_size features for LinearStrassen, in
     place, keeping weights and bias (reference model/layers.py:279-300).  With
-    square_only=False, non-square layers (and squares that are not powers of two) whose smaller
-    side is at least min_size become LinearStrassenRect instead of being skipped; below
-    min_size a layer stays an nn.Linear, i.e. a classical GEMM."""
+    square_only=False every layer whose smaller side is at least min_size becomes a
+    LinearStrassenRect instead (any shape, any number of input rows -- the reference's layer
+    refuses more than D rows); below min_size a layer stays an nn.Linear, i.e. a classical GEMM."""
     for name, child in module.named_children():
         if isinstance(child, nn.Linear) and not isinstance(child, (_LinearStrassen, LinearStrassenRect)):
-            pow2 = child.in_features & (child.in_features - 1) == 0
-            if not square_only and min(child.in_features, child.out_features) >= min_size and \
-                    not (child.in_features == child.out_features and pow2):
+            if not square_only and min(child.in_features, child.out_features) >= min_size:
                 print(f"Replacing '{name}' with LinearStrassenRect.")
                 new_layer = LinearStrassenRect(child.in_features, child.out_features,
                                                bias=child.bias is not None, device=child.weight.device,
