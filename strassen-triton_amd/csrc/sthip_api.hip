@@ -1040,7 +1040,11 @@ size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int
     const int64_t Mp = round_up(M, q), Np = round_up(N, q), Kp = round_up(K, q);
     // one level: the batch goes into a single launch, so the pre-pass buffers scale with it (and
     // only whole, tile-aligned problems take that path); deeper: batches run one after another
-    if (levels == 1) return (Mp == M && Np == N && Kp == K) ? (size_t)batch * workspace_for(Mp, Np, Kp, in_dtype, 1) : 0;
+    if (levels == 1) {
+        if (Mp != M || Np != N || Kp != K) return 0;
+        if (in_dtype == STHIP_F32) return batch == 1 ? workspace_for(Mp, Np, Kp, in_dtype, 1) : 0;   // batched-products path: one problem
+        return (size_t)batch * workspace_for(Mp, Np, Kp, in_dtype, 1);
+    }
     return workspace_for(Mp, Np, Kp, in_dtype, levels);
 }
 

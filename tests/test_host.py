@@ -53,6 +53,7 @@ def test_argument_errors_need_no_gpu():
     f32 = lambda h: 7 * 3 * h * h * 4
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == f32(512)
     assert lib.sthip_workspace_bytes(1, 1000, 1000, 1000, 0, 0, 1, 1) == 0
+    assert lib.sthip_workspace_bytes(4, 1024, 1024, 1024, 0, 0, 1, 1) == 0   # one problem per call on that path
     assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
     # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace
