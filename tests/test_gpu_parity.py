@@ -304,6 +304,50 @@ def test_fp32_batched_products(hip, monkeypatch, ta, tb, shape):
     assert rel(acc, ref + C0.double()) <= 1e-5
 
 
+def _sweep_cases():
+    import itertools
+    import random
+    rng = random.Random(20240607)
+    shapes = [(256, 256, 128), (512, 384, 256), (1024, 512, 512), (768, 1280, 512), (512, 2048, 1024),
+              (1536, 1024, 768), (2048, 2048, 1024), (640, 896, 192), (1000, 520, 264)]
+    cases = []
+    for dtype, algo, levels in itertools.product(DTYPES, ["strassen", "winograd"], [1, 2]):
+        for shape in rng.sample(shapes, 4):
+            cases.append((dtype, algo, levels, shape, rng.choice([1, 1, 3]), rng.random() < 0.5, rng.random() < 0.5,
+                          rng.random() < 0.4, rng.random() < 0.3))
+    return cases
+
+
+@pytest.mark.parametrize("dtype,algo,levels,shape,batch,ta,tb,accumulate,out_f32", _sweep_cases())
+def test_dispatch_sweep(hip, dtype, algo, levels, shape, batch, ta, tb, accumulate, out_f32):
+    """Pseudo-random walk over dtype x algorithm x levels x shape x batch x layout x accumulate x
+    result type, so that every branch of the kernel selection meets every option at least a few
+    times.  Entries in [-1, 1]: against the fp64 product the result must be exact when it is kept
+    in fp32, and equal to the correctly rounded value when every partial result is a small
+    integer; otherwise inside the dtype's tolerance."""
+    M, N, K = shape
+    lead = (batch,) if batch > 1 else ()
+    A, B = _ints(lead + (M, K), 71, -1, 1, dtype), _ints(lead + (K, N), 72, -1, 1, dtype)
+    Ag, Bg = _layout(A, ta), _layout(B, tb)
+    out_dtype = torch.float32 if (out_f32 or dtype == torch.float32) else dtype
+    exact = torch.matmul(A.double(), B.double())
+    if accumulate:
+        C0 = _ints(lead + (M, N), 73, -2, 2, out_dtype)
+        got = hip.gemm(Ag, Bg, out=C0.cuda().clone(), algo=algo, levels=levels, accumulate=True)
+        exact = exact + C0.double()
+    else:
+        got = hip.gemm(Ag, Bg, algo=algo, levels=levels, out_dtype=out_dtype)
+    assert got.dtype == out_dtype and tuple(got.shape) == tuple(exact.shape)
+    got = got.cpu().double()
+    # 16-bit intermediate products (grouped paths) hold integers up to 256 (bf16) / 2048 (fp16) exactly;
+    # quarter-size products of sums of up to four entries stay far below that for K <= 1024
+    if out_dtype == torch.float32 and (dtype == torch.float32 or K <= 512):
+        assert torch.equal(got, exact)
+    else:
+        rel = float(torch.linalg.norm(got - exact) / torch.linalg.norm(exact))
+        assert rel <= (TOL[dtype] if levels == 1 else 2 * TOL[dtype])
+
+
 def test_autograd_matmul(hip):
     A = _ints((256, 128), 31, -1, 1).cuda().requires_grad_()
     B = _ints((128, 384), 32, -1, 1).cuda().requires_grad_()
