@@ -208,7 +208,7 @@ def main():
     achieved = flops / kernel_s / 1e12
     executed = (7.0 / 8.0) ** (levels if algo != "classic" else 0)
     result = {
-        "metric": "effective TFLOP/s (2MNK/t) at 8192^2 bf16; ratio vs hipBLASLt GEMM",
+        "metric": "effective TFLOP/s (2MNK/t) at 8192\u00b2 bf16; ratio vs hipBLASLt GEMM",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": DT_NAME[dtype], "data": "synthetic",
