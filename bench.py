@@ -152,6 +152,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="strassen1_8192_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--force-tile", default=None, choices=["128x128", "128x128g", "256x128", "256x256"],
+                    help="override the library's tile table (STHIP_FORCE_TILE): 256x128 and 128x128 are the "
+                         "kernels that recombine in registers, 128x128g / 256x256 the grouped paths")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -159,6 +162,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.force_tile:
+        os.environ["STHIP_FORCE_TILE"] = args.force_tile
     if args.workload == "copy_1gib":
         copy_calibration(args.steps)
         return
@@ -214,7 +219,7 @@ def main():
         "vs_baseline": None, "dtype": DT_NAME[dtype], "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "M": M, "N": N, "K": K, "algo": algo, "levels": levels,
                    "accumulate": "fp32", "aggregate": "fp32", "out_dtype": DT_NAME[dtype],
-                   "workspace_bytes": nbytes},
+                   "workspace_bytes": nbytes, "force_tile": args.force_tile},
         "hipblaslt_tflops": round(blas_tflops, 2), "ratio_vs_hipblaslt": round(tflops / blas_tflops, 4),
         "hipblaslt_ms": round(wall_b / args.steps * 1e3, 4),
         "mfma_peak_frac": round(tflops / peak, 4),
