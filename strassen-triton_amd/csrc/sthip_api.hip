@@ -921,12 +921,9 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     const size_t es = elem_size(dt);
     if (levels == 2 && (g_stages & 8) && two_level_shape(dt, mh, nh, kh) && (!out_f32 || inner) && M == Mp && N == Np && K == Kp &&
         c_cs == 1 && c_rs % 8 == 0 && aligned_to(C, 16) && combos_ok(A, mh, kh) && combos_ok(B, kh, nh) &&
-        (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1)) {
-        const size_t flat = two_level_bytes(mh, nh, kh);
-        if (!ws || !aligned_to(ws, 256) || ws_bytes < flat)
-            return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, flat);
+        (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1) && ws && aligned_to(ws, 256) &&
+        ws_bytes >= two_level_bytes(mh, nh, kh))
         return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, stream);
-    }
     // Whole, aligned 16-bit problems: all five sums of each operand in one bandwidth-bound launch.
     const bool whole = M == Mp && N == Np && K == Kp;
     const bool vec = dt != STHIP_F32 && whole && combos_ok(A, mh, kh) && combos_ok(B, kh, nh);

@@ -44,6 +44,21 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_gemm(one, one, one, 1, 0, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == 0   # empty M
     assert lib.sthip_linear_strassen_forward(one, one, None, one, 9, 8, 0, 1, None, 0, None) == -1
     assert b"cannot be padded" in lib.sthip_last_error()
+    # two or more levels need the workspace the query asks for: refused before anything is launched
+    big = (ctypes.c_int64 * 3)(0, 1024, 1)
+    for dt in (0, 2):
+        assert lib.sthip_gemm(one, one, one, 1, 1024, 1024, 1024, big, big, big, dt, dt, 1, 2, 0, None, 0, None) == -4
+        assert b"workspace too small" in lib.sthip_last_error()
+        es = 4 if dt == 0 else 2
+        mandatory = 2 * 5 * 512 * 512 * es + 7 * 512 * 512 * 4   # sums and fp32 products of the top level
+        assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, dt, dt, 1, 2) >= mandatory
+        assert lib.sthip_gemm(one, one, one, 1, 1024, 1024, 1024, big, big, big, dt, dt, 1, 2, 0,
+                              ctypes.c_void_p(4096), mandatory - 1, None) == -4
+    assert lib.sthip_gemm(one, one, one, 1, 1024, 1024, 1024, big, big, big, 2, 2, 1, 9, 0, None, 0, None) == -5   # levels > 8
+    # an operand without a unit stride is a layout error
+    bad = (ctypes.c_int64 * 3)(0, 2048, 2)
+    assert lib.sthip_gemm(one, one, one, 1, 64, 64, 64, bad, big, big, 2, 2, 1, 1, 0, None, 0, None) == -3
+    assert b"no unit stride" in lib.sthip_last_error()
     # workspace.  One level: room for the ten quadrant sums (5 per operand) and the parked accumulator when the shape is
     # tile aligned, per batch entry; nothing for fp32, odd or unaligned shapes, or classic.
     sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles)
