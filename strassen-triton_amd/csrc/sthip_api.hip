@@ -336,11 +336,9 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         const int64_t sa_bs = (int64_t)(sa_b / 2), sb_bs = (int64_t)(sb_b / 2);
         auto SAo = [&](int o) { return (const void*)(SA + (size_t)o * batch * sa_b); };
         auto SBo = [&](int o) { return (const void*)(SB + (size_t)o * batch * sb_b); };
-        auto rawA = [&](int q) { return Seg2{Aq[q], nullptr, a_ld, 0, a_bs, 0}; };
         auto set = [&](int i, const void* a, int64_t ald, int64_t abs_, const void* b, int64_t bld, int64_t bbs) {
             p.seg[i] = {a, b, ald, bld, abs_, bbs};
         };
-        (void)rawA;
         if (algo == STHIP_STRASSEN) {
             // kernel order M3 M6 M5 M7 M1 M2 M4; A sums S2 S3 S5 S7 S9 = outputs 0..4, B sums S1 S4 S6 S8 S10
             set(0, Aq[0], a_ld, a_bs, SBo(0), sb_ld, sb_bs);      // M3 = A11 S1

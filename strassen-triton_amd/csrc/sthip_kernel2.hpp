@@ -24,8 +24,9 @@
 
 namespace sthip {
 
-// Experiment switches for the micro-benchmarks (always 0 in the library):
-// 1 = skip the global->LDS loads, 2 = skip the workgroup barrier, 4 = skip the fragment reads.
+// Experiment switches for kernel4_microbench.hip (always 0 in the library):
+// 1 = skip the global->LDS loads, 2 = skip the workgroup barrier, 4 = skip the fragment reads,
+// 64 = skip the MFMAs.
 #ifndef STHIP_DBG
 #define STHIP_DBG 0
 #endif
