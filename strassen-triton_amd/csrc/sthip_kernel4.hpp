@@ -12,6 +12,11 @@
 // so that the chip works through one product at a time and each behaves like a classical GEMM.
 // The recombination of the seven outputs is a separate elementwise pass.
 //
+// Matrix instruction: v_mfma_f32_16x16x32 (a 128 x 128 wave tile is 8 x 8 of them per 32 k).
+// Sustained matrix throughput on this card is set by the power limit, and with random operands
+// the 16x16x32 form sustains 14 % more than 32x32x16 in a register-only loop (2.08 against 1.82
+// PFLOP/s); in this kernel it is worth 1 - 4 %.
+//
 // Pipeline: k-steps of 64 (whole 128-byte lines per row), two LDS stages of 64 KiB, the
 // barrier of a step sits just before the next step's first fragments are read, at which
 // point the current stage is free and is refilled with the step two ahead.
@@ -33,12 +38,12 @@ constexpr int kSmemBytes4 = kStages4 * kStageBytes4;     // 128 KiB
 
 // A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 64 w + 8 i + L/8, i = 0..7,
 // chunk (L%8) ^ ((row/2)%8).  n-contiguous B: 64 k-rows x 32 chunks (512 bytes); wave w loads
-// k-rows 16 w + 2 i + L/32, i = 0..7, chunk (L%32) ^ ((k%4)*4).
+// k-rows 16 w + 2 i + L/32, i = 0..7, chunk (L%32) ^ ((k%4)*4) ^ (((k/8)%2)*2).
 template <bool B_KC>
 struct Loader4 {
     const char* a_base; const char* b_base;
     int64_t a_row_bytes, b_row_bytes, a_step_bytes, b_step_bytes;
-    uint32_t a_voff[2], b_voff[2];
+    uint32_t a_voff[2], b_voff[4];   // b: index (i % 2) + 2 (i / 4) of the wave's load i
     int seg, kt, total_seg, KT;
     int batch, tile_m, tile_n, wave;
     const Gemm2Params* P;
@@ -58,16 +63,18 @@ struct Loader4 {
             b_base = b + (int64_t)(tile_n + wave * 64) * s.b_ld * 2;
             b_row_bytes = 8 * s.b_ld * 2;
             b_step_bytes = kBK4 * 2;
-            b_voff[0] = (uint32_t)(((lane >> 3) * s.b_ld + chunk0 * 8) * 2);
-            b_voff[1] = (uint32_t)(((lane >> 3) * s.b_ld + (chunk0 ^ 4) * 8) * 2);
+            b_voff[0] = b_voff[2] = (uint32_t)(((lane >> 3) * s.b_ld + chunk0 * 8) * 2);
+            b_voff[1] = b_voff[3] = (uint32_t)(((lane >> 3) * s.b_ld + (chunk0 ^ 4) * 8) * 2);
         } else {
-            // k%4 = 2 (i%2) + L/32
+            // k-row of load i: k = 16 w + 2 i + L/32, so k%4 = 2 (i%2) + L/32 and (k/8)%2 = i/4;
+            // the chunk stored in slot s of row k is s ^ ((k%4) * 4) ^ (((k/8)%2) * 2)
             const int chunk = (lane & 31) ^ ((lane >> 5) << 2);
             b_base = b + ((int64_t)(wave * 16) * s.b_ld + tile_n) * 2;
             b_row_bytes = 2 * s.b_ld * 2;
             b_step_bytes = (int64_t)kBK4 * s.b_ld * 2;
-            b_voff[0] = (uint32_t)(((lane >> 5) * s.b_ld + chunk * 8) * 2);
-            b_voff[1] = (uint32_t)(((lane >> 5) * s.b_ld + (chunk ^ 8) * 8) * 2);
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                b_voff[v] = (uint32_t)(((lane >> 5) * s.b_ld + (chunk ^ ((v & 1) << 3) ^ ((v >> 1) << 1)) * 8) * 2);
         }
     }
 
@@ -77,7 +84,7 @@ struct Loader4 {
 #pragma unroll
         for (int i = 0; i < 8; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], sb + i * 1024);
+        for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[(i & 1) | ((i >> 2) << 1)], sb + i * 1024);
         a_base += a_step_bytes;
         b_base += b_step_bytes;
         if (++kt == KT) {
@@ -89,13 +96,30 @@ struct Loader4 {
     __device__ __forceinline__ bool done() const { return seg >= total_seg; }
 };
 
-// n-contiguous B tile with 512-byte k-rows: same transposing read as the narrower tiles.
-__device__ __forceinline__ u32x4 read_frag4_mc(const char* tile, int sub, int kg) {
+// Operand fragments of v_mfma_f32_16x16x32: lane L holds, for row (or column) L % 16 of a
+// 16-wide block, the eight k-values 8 (L / 16) .. + 7 of a group of 32.
+//
+// k-contiguous tile (128-byte rows, 16-byte chunks XOR-swizzled with (row/2)%8): one 16-byte read
+// per lane.  A 16-lane group reads 16 rows at one chunk position: rows r, r+1 share a slot but lie
+// 128 bytes apart, so the group covers all 64 banks once.
+__device__ __forceinline__ u32x4 read_frag16_kc(const char* tile, int sub, int kg) {
+    const int lane = threadIdx.x & 63;
+    const int row = sub + (lane & 15);
+    const int slot = (kg * 4 + (lane >> 4)) ^ ((row >> 1) & 7);
+    return *reinterpret_cast<const u32x4*>(tile + row * 128 + slot * 16);
+}
+
+// n-contiguous B tile (64 k-rows of 512 bytes): two transposing reads.  In each 16-lane group,
+// lane r addresses 4 consecutive n of k-row k0 + r/4 (k0 = 32 kg + 8 group) at n = sub + 4 (r%4);
+// the read hands lane i the four k-values k0..k0+3 of column sub + i; the second read does
+// k0+4..k0+7.  The slot swizzle flips bit 1 with (k/8)%2 so that groups 0/1 (and 2/3) use
+// disjoint banks.
+__device__ __forceinline__ u32x4 read_frag16_mc(const char* tile, int sub, int kg) {
     const int lane = threadIdx.x & 63;
     const int l16 = lane & 15, grp = lane >> 4;
-    const int k = kg * 16 + (grp >> 1) * 8 + (l16 >> 2);
-    const int chunk = (sub >> 3) + (grp & 1) * 2 + ((l16 & 3) >> 1);
-    const int slot = chunk ^ (((l16 >> 2) & 3) << 2);
+    const int k = kg * 32 + grp * 8 + (l16 >> 2);
+    const int chunk = (sub >> 3) + ((l16 & 3) >> 1);
+    const int slot = chunk ^ (((l16 >> 2) & 3) << 2) ^ ((grp & 1) << 1);
     const char* p = tile + k * 512 + slot * 16 + (l16 & 1) * 8;
     typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
@@ -105,15 +129,27 @@ __device__ __forceinline__ u32x4 read_frag4_mc(const char* tile, int sub, int kg
     return r;
 }
 
-struct Acc4 {   // one 128 x 128 wave tile = 4 x 4 MFMA tiles = 256 registers
-    f32x16 t[4][4];
+// acc (16 n x 16 m, transposed so that a lane holds four consecutive n) += B-fragment x A-fragment.
+// Written as assembly so that the accumulator is updated in place: given the builtin, the
+// register allocator puts result and addend in different registers and permutes the 64
+// accumulators back with ~180 register copies per k-step.
+template <class T>
+__device__ __forceinline__ void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b) {
+    if constexpr (__is_same(T, bf16_t))
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+    else
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+struct Acc4 {   // one 128 x 128 wave tile = 8 x 8 MFMA tiles = 256 registers
+    f32x4 t[8][8];
     __device__ __forceinline__ void zero() {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 8; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) t[i][j][e] = 0.f;
+                for (int e = 0; e < 4; ++e) t[i][j][e] = 0.f;
     }
 };
 
@@ -124,17 +160,17 @@ struct Pipe4 {
     uint32_t smem_addr;
     int g, total, slot;
     int wm, wn;
-    u32x4 fa[2][4], fb[2][4];
+    u32x4 fa[2][8], fb[2][8];   // [buffer][16-wide block]: fragments of one group of 32 k
 
     __device__ __forceinline__ void read_frags(int buf, int sl, int kg) {
         const char* s = smem + sl * kStageBytes4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if constexpr (B_KC) fb[buf][j] = read_frag2<true>(s + kATile4, wn + j * 32, kg);
-            else fb[buf][j] = read_frag4_mc(s + kATile4, wn + j * 32, kg);
+        for (int j = 0; j < 8; ++j) {
+            if constexpr (B_KC) fb[buf][j] = read_frag16_kc(s + kATile4, wn + j * 16, kg);
+            else fb[buf][j] = read_frag16_mc(s + kATile4, wn + j * 16, kg);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa[buf][i] = read_frag2<true>(s, wm + i * 32, kg);
+        for (int i = 0; i < 8; ++i) fa[buf][i] = read_frag16_kc(s, wm + i * 16, kg);
     }
 
     __device__ __forceinline__ void start() {
@@ -144,7 +180,7 @@ struct Pipe4 {
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i] = u32x4{0, 0, 0, 0}; }
+                for (int i = 0; i < 8; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i] = u32x4{0, 0, 0, 0}; }
         }
         if (!(STHIP_DBG & 1)) {
             ld.issue(smem_addr);
@@ -158,10 +194,10 @@ struct Pipe4 {
     __device__ __forceinline__ void run(Acc4& acc, int KT) {
         for (int kt = 0; kt < KT; ++kt, ++g) {
 #pragma unroll
-            for (int kg = 0; kg < 4; ++kg) {
-                const int nb = (kg + 1) & 1, cb = kg & 1;
-                if (kg < 3) {
-                    if (!(STHIP_DBG & 4)) read_frags(nb, slot, kg + 1);
+            for (int kg = 0; kg < 2; ++kg) {
+                const int nb = kg ^ 1, cb = kg;
+                if (kg == 0) {
+                    if (!(STHIP_DBG & 4)) read_frags(nb, slot, 1);
                 } else {
                     // Every wave has read all fragments of this step: after the barrier its stage is
                     // free for the step two ahead.  Step g+1 (the only load batch in flight) must
@@ -172,65 +208,59 @@ struct Pipe4 {
                     if (!(STHIP_DBG & 4) && g + 1 < total) read_frags(nb, slot ^ 1, 0);
                 }
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < 8; ++i)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (!(STHIP_DBG & 64)) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
-                if (!(STHIP_DBG & (4 | 64))) {
-#pragma unroll
-                    for (int m = 0; m < 16; ++m) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-                    }
-                }
+                    for (int j = 0; j < 8; ++j)
+                        if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                 __builtin_amdgcn_sched_barrier(0);
             }
             slot ^= 1;
         }
+        // the matrix instructions are opaque to the compiler's hazard checks: let the last results
+        // retire before the epilogue reads the accumulators
+        asm volatile("s_nop 15\n\ts_nop 15");
     }
 };
 
+// Lane l of MFMA tile (i, j) holds m = 16 i + l % 16 and n = 16 j + 4 (l / 16) + 0..3.
 template <class T>
 __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& P, char* Cb, int quad, int row, int col) {
     const int lane = threadIdx.x & 63;
     const int esz = P.out_f32 ? 4 : 2;
-    const int m0 = (quad >> 1) * P.Mh + row + (lane & 31);
-    const int n0 = (quad & 1) * P.Nh + col + 4 * (lane >> 5);
+    const int m0 = (quad >> 1) * P.Mh + row + (lane & 15);
+    const int n0 = (quad & 1) * P.Nh + col + 4 * (lane >> 4);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 8; ++j) {
+            float v[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc.t[i][j][4 * g + e];
-                char* dst = Cb + ((int64_t)(m0 + i * 32) * P.c_rs + (n0 + j * 32 + 8 * g)) * esz;
-                if (P.out_f32) {
-                    f32x4* d = reinterpret_cast<f32x4*>(dst);
-                    f32x4 o = {v[0], v[1], v[2], v[3]};
-                    if (P.accumulate) o += *d;
-                    *d = o;
-                } else {
-                    u32x2* d = reinterpret_cast<u32x2*>(dst);
-                    if (P.accumulate) {
-                        const u32x2 old = *d;
-                        const uint32_t w0 = old[0], w1 = old[1];
-                        if constexpr (__is_same(T, bf16_t)) {
-                            v[0] += bf16lo(w0); v[1] += bf16hi(w0); v[2] += bf16lo(w1); v[3] += bf16hi(w1);
-                        } else {
-                            const f16x2 h0 = as_f16x2(w0), h1 = as_f16x2(w1);
-                            v[0] += (float)h0[0]; v[1] += (float)h0[1]; v[2] += (float)h1[0]; v[3] += (float)h1[1];
-                        }
+            for (int e = 0; e < 4; ++e) v[e] = acc.t[i][j][e];
+            char* dst = Cb + ((int64_t)(m0 + i * 16) * P.c_rs + (n0 + j * 16)) * esz;
+            if (P.out_f32) {
+                f32x4* d = reinterpret_cast<f32x4*>(dst);
+                f32x4 o = {v[0], v[1], v[2], v[3]};
+                if (P.accumulate) o += *d;
+                *d = o;
+            } else {
+                u32x2* d = reinterpret_cast<u32x2*>(dst);
+                if (P.accumulate) {
+                    const u32x2 old = *d;
+                    const uint32_t w0 = old[0], w1 = old[1];
+                    if constexpr (__is_same(T, bf16_t)) {
+                        v[0] += bf16lo(w0); v[1] += bf16hi(w0); v[2] += bf16lo(w1); v[3] += bf16hi(w1);
+                    } else {
+                        const f16x2 h0 = as_f16x2(w0), h1 = as_f16x2(w1);
+                        v[0] += (float)h0[0]; v[1] += (float)h0[1]; v[2] += (float)h1[0]; v[3] += (float)h1[1];
                     }
-                    u32x2 o;
-                    if constexpr (__is_same(T, bf16_t)) { o[0] = pack_bf16(v[0], v[1]); o[1] = pack_bf16(v[2], v[3]); }
-                    else { o[0] = pack_f16(v[0], v[1]); o[1] = pack_f16(v[2], v[3]); }
-                    *d = o;
                 }
-                if (g == 3) __builtin_amdgcn_sched_barrier(0);
+                u32x2 o;
+                if constexpr (__is_same(T, bf16_t)) { o[0] = pack_bf16(v[0], v[1]); o[1] = pack_bf16(v[2], v[3]); }
+                else { o[0] = pack_f16(v[0], v[1]); o[1] = pack_f16(v[2], v[3]); }
+                *d = o;
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
