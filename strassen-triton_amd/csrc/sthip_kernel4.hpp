@@ -93,6 +93,23 @@ struct Loader4 {
         }
     }
 
+    // Load q (0..7 the A tile, 8..15 the B tile) of the next k-step; advance() after the sixteenth.
+    __device__ __forceinline__ void issue_one(uint32_t stage_addr, int q) {
+        if (q < 8) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], stage_addr + wave * 8192 + q * 1024);
+        else {
+            const int i = q - 8;
+            lds_dma16(b_base + i * b_row_bytes, b_voff[(i & 1) | ((i >> 2) << 1)], stage_addr + kATile4 + wave * 8192 + i * 1024);
+        }
+    }
+    __device__ __forceinline__ void advance() {
+        a_base += a_step_bytes;
+        b_base += b_step_bytes;
+        if (++kt == KT) {
+            kt = 0;
+            if (++seg < total_seg) point_at_segment();
+        }
+    }
+
     __device__ __forceinline__ bool done() const { return seg >= total_seg; }
 };
 
@@ -162,15 +179,16 @@ struct Pipe4 {
     int wm, wn;
     u32x4 fa[2][8], fb[2][8];   // [buffer][16-wide block]: fragments of one group of 32 k
 
-    __device__ __forceinline__ void read_frags(int buf, int sl, int kg) {
+    // The A and the B fragment of 16-wide block r.
+    __device__ __forceinline__ void read_pair(int buf, int sl, int kg, int r) {
         const char* s = smem + sl * kStageBytes4;
+        if constexpr (B_KC) fb[buf][r] = read_frag16_kc(s + kATile4, wn + r * 16, kg);
+        else fb[buf][r] = read_frag16_mc(s + kATile4, wn + r * 16, kg);
+        fa[buf][r] = read_frag16_kc(s, wm + r * 16, kg);
+    }
+    __device__ __forceinline__ void read_frags(int buf, int sl, int kg) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if constexpr (B_KC) fb[buf][j] = read_frag16_kc(s + kATile4, wn + j * 16, kg);
-            else fb[buf][j] = read_frag16_mc(s + kATile4, wn + j * 16, kg);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) fa[buf][i] = read_frag16_kc(s, wm + i * 16, kg);
+        for (int r = 0; r < 8; ++r) read_pair(buf, sl, kg, r);
     }
 
     __device__ __forceinline__ void start() {
@@ -196,23 +214,40 @@ struct Pipe4 {
 #pragma unroll
             for (int kg = 0; kg < 2; ++kg) {
                 const int nb = kg ^ 1, cb = kg;
-                if (kg == 0) {
-                    if (!(STHIP_DBG & 4)) read_frags(nb, slot, 1);
-                } else {
+                if (kg == 1) {
                     // Every wave has read all fragments of this step: after the barrier its stage is
                     // free for the step two ahead.  Step g+1 (the only load batch in flight) must
                     // have landed before its fragments are read.
                     if (!(STHIP_DBG & 1)) wait_vmcnt_imm<0>();
                     if (!(STHIP_DBG & 2)) __syncthreads();
-                    if (!(STHIP_DBG & 1) && !ld.done()) ld.issue(smem_addr + slot * kStageBytes4);
-                    if (!(STHIP_DBG & 4) && g + 1 < total) read_frags(nb, slot ^ 1, 0);
                 }
+                // The sixteen loads of step g+2 go out four per row over the first four rows of matrix
+                // instructions (measured at 8192^3: all sixteen at once 0.953 ms, eight per row 0.925,
+                // four 0.900, two 0.917).
+                const bool issuing = kg == 1 && !(STHIP_DBG & 1) && !ld.done();
+                // Fragments of the next k-group come in between the rows of matrix instructions, one
+                // A and one B fragment (two or three LDS reads) per row: few enough in flight for the
+                // LDS counter (4 bits) to tell the old fragments from the new -- with all 24 reads
+                // issued first, the first matrix instruction waited for ten of them.  In the last
+                // step the "next" fragments are stale data that nobody uses.
+                const int nsl = kg == 0 ? slot : slot ^ 1, nkg = kg ^ 1;
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
+                for (int i = 0; i < 8; ++i) {
+                    if (issuing && i < 4) {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j)
+                        for (int q = 0; q < 4; ++q) ld.issue_one(smem_addr + slot * kStageBytes4, 4 * i + q);
+                        if (i == 3) ld.advance();
+                    }
+                    if (!(STHIP_DBG & 4)) {
+                        read_pair(nb, nsl, nkg, i);
+                    }
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) {
+                        const int j = (i & 1) ? 7 - jj : jj;   // boustrophedon: the B fragment carries over between rows
                         if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
-                __builtin_amdgcn_sched_barrier(0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             slot ^= 1;
         }
