@@ -171,6 +171,34 @@ def test_replace_linear_with_strassen_rect(capsys):
     assert O.rel_fro(net(x).cpu(), before.cpu()) <= 1e-5
 
 
+@pytest.mark.parametrize("levels,n", [(1, 1024), (2, 1024), (1, 384)])
+def test_calls_can_be_captured_in_a_hip_graph(levels, n):
+    """The C ABI only enqueues kernels on the stream it is given (no allocation, no memset, no
+    synchronisation), so a call with caller-owned output and workspace can be captured into a HIP
+    graph.  Every replay, with new operand values written in place and eager work in between, must
+    reproduce the eager result bit for bit."""
+    import strassen_hip
+    g = torch.Generator().manual_seed(11)
+    A = torch.randn(n, n, generator=g).to(torch.bfloat16).cuda()
+    B = torch.randn(n, n, generator=g).to(torch.bfloat16).cuda()
+    out = torch.empty(n, n, dtype=torch.bfloat16, device="cuda")
+    ws = torch.empty(max(1, strassen_hip.workspace_bytes(A, B, levels=levels)), dtype=torch.uint8, device="cuda")
+    strassen_hip.gemm(A, B, out, levels=levels, workspace=ws)          # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        strassen_hip.gemm(A, B, out, levels=levels, workspace=ws)
+    for rep in range(3):
+        A.copy_(torch.randn(n, n, generator=g).to(torch.bfloat16))
+        B.copy_(torch.randn(n, n, generator=g).to(torch.bfloat16))
+        eager = strassen_hip.gemm(A, B, levels=levels)
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+
+
 def test_cpu_tensors_are_refused():
     import fixed_strassen
     with pytest.raises(RuntimeError, match="no CPU implementation"):
