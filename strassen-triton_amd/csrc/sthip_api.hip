@@ -302,6 +302,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2);
         char* SA = ws;                                // [5][batch] blocks of Mh x Kh (storage order of A)
         char* SB = ws + (size_t)batch * 5 * sa_b;
+        // region after the sums: parked fp32 tiles (256 x 128 kernel) or the seven 16-bit products (grouped paths)
         p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
         const int nout = algo == STHIP_STRASSEN ? 5 : 4;
