@@ -27,11 +27,16 @@ _DTYPES = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
 # (N, depth) grid of reference main_profiling.py:250-261.
 _GRID = [(1024, 1), (1024, 2), (2048, 1), (2048, 2), (4096, 1), (4096, 2),
          (8192, 1), (8192, 2), (8192, 3), (16384, 1), (16384, 2), (16384, 3),
-         (32768, 1), (32768, 2), (32768, 3), (32768, 4)]
+         (32768, 1), (32768, 2), (32768, 3), (32768, 4),
+         # beyond the reference's grid: where more levels start to pay on this machine
+         (65536, 1), (65536, 2), (65536, 3)]
 
 
 def _runs_for(n: int) -> tuple[int, int]:
-    """(warm-up, timed calls) per problem size (reference main_profiling.py:279-289)."""
+    """(warm-up, timed calls) per problem size (reference main_profiling.py:279-289; fewer for
+    the sizes where one call takes tens of milliseconds or more)."""
+    if n >= 32768:
+        return 3, 10
     if n >= 4096:
         return 10, 50
     if n >= 1024:
