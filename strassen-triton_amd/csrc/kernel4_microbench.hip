@@ -6,7 +6,8 @@
 //   ./kernel4_microbench [n = 8192] [leading-dimension padding in elements = 0]
 //
 // STHIP_DBG bits: 1 = no global -> LDS loads, 2 = no workgroup barrier, 4 = no LDS fragment reads
-// (MFMAs then run on zeros), 64 = no MFMAs.  0 is the kernel as shipped; 5 is MFMAs alone.
+// (MFMAs then run on zeros), 8 = no store of the tile, 16 = the kernel returns at once (launch and
+// dispatch alone), 64 = no MFMAs.  0 is the kernel as shipped; 5 is MFMAs alone.
 // Results are timings only: with any bit set the product is not computed.
 #include <hip/hip_runtime.h>
 #include <stdio.h>
@@ -26,7 +27,7 @@ template <bool BKC> void run(int n, int pad) {
   CK(hipMemcpy(A, h.data(), bytes, hipMemcpyHostToDevice)); CK(hipMemcpy(B, h.data(), bytes, hipMemcpyHostToDevice));
   Gemm2Params p; memset(&p, 0, sizeof(p));
   p.seg[0] = {A, B, ld, ld, 0, 0};
-  p.C = C; p.c_rs = ld; p.Mh = n; p.Nh = n; p.Kh = n; p.tiles_m = n / 256; p.tiles_n = n / 256; p.group_m = 4; p.nprod = 1;
+  p.C = C; p.c_rs = ld; p.Mh = n; p.Nh = n; p.Kh = n; p.tiles_m = n / 256; p.tiles_n = n / 256; p.group_m = 4; p.nprod = 1; p.c_wide = (ld % 8 == 0);
   auto kern = gemm4_kernel<bf16_t, BKC>;
   CK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes4));
   dim3 grid(p.tiles_m * p.tiles_n, 1);

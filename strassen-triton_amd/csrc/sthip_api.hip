@@ -81,6 +81,10 @@ static int forced_tile() {
 }
 
 static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+// 16-bit C whose rows, product stride and batch stride keep 16-byte alignment (strides in elements)
+static int wide_rows(const void* C, int64_t rs, int64_t ps, int64_t bs) {
+    return aligned_to(C, 16) && rs % 8 == 0 && ps % 8 == 0 && bs % 8 == 0 ? 1 : 0;
+}
 
 // ------------------------------------------------------------------ quadrant-sum pre-pass
 // out[o] = sum_q coef[o][q] * quadrant q, for up to five outputs at once, on matrices seen
@@ -404,6 +408,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             if (pick == 4) {
                 p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
                 p.group_m = 4;
+                p.c_wide = wide_rows(p.C, p.c_rs, p.c_ps, p.c_bs);
                 e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
             } else {
                 const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
@@ -426,6 +431,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     if (pick == 4) {
         p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
         p.group_m = 4; p.nprod = 1;
+        p.c_wide = wide_rows(p.C, p.c_rs, 0, p.c_bs);
         e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
     } else if (pick == 3) {
         p.tiles_m = (int)(Mh / kBM3);
@@ -765,6 +771,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     hipError_t e;
     if (big) {
         g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
+        g.c_wide = wide_rows(g.C, g.c_rs, g.c_ps, 0);
         e = t4->fn[b_kc ? 1 : 0](g, 1, stream);
     } else {
         const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);

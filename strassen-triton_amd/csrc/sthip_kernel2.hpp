@@ -54,6 +54,7 @@ struct Gemm2Params {
     int Mh, Nh, Kh;       // extent of one segment product
     int tiles_m, tiles_n;
     int out_f32, accumulate, group_m;
+    int c_wide;           // 256 x 256 kernel: C, its rows and its product / batch strides are 16-byte aligned
 };
 
 __device__ __forceinline__ void wait_vmcnt(int n) {

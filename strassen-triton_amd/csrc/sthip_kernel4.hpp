@@ -299,9 +299,47 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
     }
 }
 
+// The 16-bit, non-accumulating store, staged through LDS so that every store instruction writes
+// four rows x 256 contiguous bytes (16 bytes per lane) instead of sixteen rows x 32 bytes: with
+// all workgroups of a round storing at once, the partial-line pattern of the MFMA layout costs
+// about twice the time.  Each wave uses its own 32 KiB of the (now idle) stage buffers: row r of
+// its 128 x 128 tile at r * 256, the 8-byte chunk c of a row at ((c ^ 2 (r % 16)) * 8, which
+// spreads the sixteen rows a write instruction touches over all banks and keeps 16-byte chunks
+// whole for the read back.  The caller has synchronised the workgroup.
+template <class T>
+__device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Params& P, char* Cb, char* smem,
+                                                int wave, int row, int col) {
+    const int lane = threadIdx.x & 63;
+    const int l16 = lane & 15, q = lane >> 4;
+    char* w = smem + wave * 32768;
+    uint32_t waddr[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) waddr[j] = l16 * 256 + (((4 * j + q) ^ (2 * l16)) * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            u32x2 o;
+            if constexpr (__is_same(T, bf16_t)) { o[0] = pack_bf16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_bf16(acc.t[i][j][2], acc.t[i][j][3]); }
+            else { o[0] = pack_f16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_f16(acc.t[i][j][2], acc.t[i][j][3]); }
+            *reinterpret_cast<u32x2*>(w + i * 4096 + waddr[j]) = o;
+        }
+    }
+    // read back: lane -> row 4 r + q, 16-byte chunk l16; the same wave wrote it, LDS keeps order
+    char* dst = Cb + ((int64_t)(row + q) * P.c_rs + (col + 8 * l16)) * 2;
+    const int64_t step = (int64_t)4 * P.c_rs * 2;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+        const int rr = 4 * (r & 3) + q;                       // (4 r + q) % 16
+        const u32x4 v = *reinterpret_cast<const u32x4*>(w + (4 * r + q) * 256 + ((l16 ^ rr) * 16));
+        *reinterpret_cast<u32x4*>(dst + r * step) = v;
+    }
+}
+
 template <class T, bool B_KC>
 __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    if (STHIP_DBG & 16) return;
     // blockIdx.x = product * tiles + tile: the XCD-aware renumbering works within one product
     const int tiles = P.tiles_m * P.tiles_n;
     const int prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
@@ -331,7 +369,13 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     Acc4 r;
     r.zero();
     pipe.run(r, KT);
-    store_tile4<T>(r, P, Cb, 0, tile_m + pipe.wm, tile_n + pipe.wn);
+    if (STHIP_DBG & 8) return;
+    if (P.c_wide && !P.out_f32 && !P.accumulate && !(STHIP_DBG & 32)) {
+        __syncthreads();   // every wave has read its last fragments: the stage buffers are free
+        store_tile4_lds<T>(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
+    } else {
+        store_tile4<T>(r, P, Cb, 0, tile_m + pipe.wm, tile_n + pipe.wn);
+    }
 }
 
 }  // namespace sthip

@@ -377,3 +377,22 @@ def test_every_pipelined_tile_exact(hip, monkeypatch, tile, dtype, algo, tb):
     assert torch.equal(Cacc.cpu().double(), C0.double() + want)
     Cn = hip.gemm(A[0, :, :128].contiguous().cuda(), _layout(B[0, :128], tb), algo=algo, levels=1)   # |C| <= 128: exact in 16 bit
     assert Cn.dtype == dtype and torch.equal(Cn.cpu().double(), A[0, :, :128].double() @ B[0, :128].double())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("pad,off", [(0, 0), (8, 0), (4, 0), (8, 4)])
+@pytest.mark.parametrize("algo,levels", [("classic", 0), ("strassen", 1)])
+def test_large_tile_store_alignment(hip, monkeypatch, dtype, pad, off, algo, levels):
+    """The 256 x 256 kernel stores 16-bit results sixteen bytes per lane when C, its rows and its
+    strides are 16-byte aligned, eight bytes per lane otherwise: results written into a view of a
+    wider buffer (row stride N + pad, first column off) are exact either way and the columns
+    outside the view stay untouched."""
+    monkeypatch.setenv("STHIP_FORCE_TILE", "256x256")
+    M, N, K = 1024, 512, 128
+    A, B = _ints((M, K), 61, -1, 1, dtype), _ints((K, N), 62, -1, 1, dtype)   # |C| <= 128: exact in 16 bit
+    want = A.double() @ B.double()
+    buf = torch.full((M, N + pad + off), 7.0, dtype=dtype, device="cuda")
+    out = buf[:, off:off + N]
+    hip.gemm(A.cuda(), B.cuda(), out=out, algo=algo, levels=levels)
+    assert torch.equal(out.cpu().double(), want)
+    assert torch.all(buf[:, :off] == 7) and torch.all(buf[:, off + N:] == 7)
