@@ -7,7 +7,8 @@
 //
 // STHIP_DBG bits: 1 = no global -> LDS loads, 2 = no workgroup barrier, 4 = no LDS fragment reads
 // (MFMAs then run on zeros), 8 = no store of the tile, 16 = the kernel returns at once (launch and
-// dispatch alone), 64 = no MFMAs.  0 is the kernel as shipped; 5 is MFMAs alone.
+// dispatch alone), 32 = the 8-byte store straight from the accumulators, 64 = no MFMAs, 128 = every
+// k-step loads the first k-slice again (loads that hit in cache).  0 is the kernel as shipped; 5 is MFMAs alone.
 // Results are timings only: with any bit set the product is not computed.
 #include <hip/hip_runtime.h>
 #include <stdio.h>

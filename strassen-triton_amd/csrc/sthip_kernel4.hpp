@@ -85,12 +85,7 @@ struct Loader4 {
         for (int i = 0; i < 8; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
 #pragma unroll
         for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[(i & 1) | ((i >> 2) << 1)], sb + i * 1024);
-        a_base += a_step_bytes;
-        b_base += b_step_bytes;
-        if (++kt == KT) {
-            kt = 0;
-            if (++seg < total_seg) point_at_segment();
-        }
+        advance();
     }
 
     // Load q (0..7 the A tile, 8..15 the B tile) of the next k-step; advance() after the sixteenth.
@@ -102,8 +97,10 @@ struct Loader4 {
         }
     }
     __device__ __forceinline__ void advance() {
-        a_base += a_step_bytes;
-        b_base += b_step_bytes;
+        if (!(STHIP_DBG & 128)) {   // bit 128: every k-step loads the first one again (cache hits)
+            a_base += a_step_bytes;
+            b_base += b_step_bytes;
+        }
         if (++kt == KT) {
             kt = 0;
             if (++seg < total_seg) point_at_segment();
