@@ -14,8 +14,9 @@
 namespace sthip {
 
 static thread_local char g_err[512] = "";
-// Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM.
-// Only the profiling hook sthip_debug_set_stages changes it.
+// Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
+// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch.  Only the
+// profiling hook sthip_debug_set_stages changes it.
 static int g_stages = 15;
 
 static int fail(int code, const char* fmt, ...) {
