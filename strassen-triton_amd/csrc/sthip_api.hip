@@ -66,7 +66,7 @@ static const LaunchTable3* table3_for(int dt, int algo) {
 }
 
 static const LaunchTable3* table4_for(int dt) {
-    return dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
+    return dt == STHIP_F32 ? &kLaunch4_0 : dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
 }
 
 // STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 overrides the tile table where the shape allows
@@ -454,6 +454,8 @@ static size_t f32_batched_bytes(int64_t Mh, int64_t Nh, int64_t Kh) {
 }
 static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
                                  bool accumulate, char* ws, hipStream_t stream);
+static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
+                                 bool accumulate, char* ws, hipStream_t stream);
 
 static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                         int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
@@ -508,6 +510,28 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         int rc = launch_pipelined(A, B, C, c_rs, batch, a_bs, b_bs, c_bs, Mh, Nh, Kh, dt, out_f32, algo, accumulate,
                                   a_kc, b_kc, ws, ws_bytes, stream);
         if (rc <= 0) return rc;
+    }
+    // fp32 on the 256 x 256 pipelined kernel (A contiguous along k, enough tiles to fill the chip):
+    // a classical product directly; one Strassen level as sums, ONE grouped launch of the seven
+    // products and the recombination pass.  Measured at 8192^3: the classical product runs at
+    // 142 TFLOP/s against 85 on the fused kernel.
+    if (fast && dt == STHIP_F32 && a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && Kh % 32 == 0 && forced_tile() != 2) {
+        const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch;
+        if (!split && tiles4 >= 224) {
+            Gemm2Params g;
+            memset(&g, 0, sizeof(g));
+            g.seg[0] = Seg2{A.p, B.p, A.rs, b_kc ? B.cs : B.rs, a_bs, b_bs};
+            g.C = C; g.c_rs = c_rs; g.c_bs = c_bs;
+            g.Mh = (int)Mh; g.Nh = (int)Nh; g.Kh = (int)Kh;
+            g.tiles_m = (int)(Mh / kBM4); g.tiles_n = (int)(Nh / kBN4);
+            g.out_f32 = 1; g.accumulate = accumulate ? 1 : 0; g.group_m = 4; g.nprod = 1;
+            hipError_t e = table4_for(dt)->fn[b_kc ? 1 : 0](g, (int)batch, stream);
+            if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+            return STHIP_OK;
+        }
+        if (algo == STHIP_STRASSEN && batch == 1 && 7 * tiles4 >= 224 && ws && aligned_to(ws, 256) &&
+            ws_bytes >= f32_batched_bytes(Mh, Nh, Kh))
+            return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, stream);
     }
     // fp32, one Strassen level: run the seven products side by side as a batch (see
     // one_level_f32_batched).  Measured against the fused kernel: 5 x faster at 1024^3 (one product
@@ -613,10 +637,11 @@ static int check_launch(const char* what) {
 // All quadrant sums of one operand in one launch (see quad_combos_kernel).  X is the operand,
 // (r_blk, c_blk) the block size in its logical (row, col) indexing; outputs are dense blocks in
 // the storage orientation of X, `out_stride` bytes apart.
-static bool combos_ok(View X, int64_t r_blk, int64_t c_blk) {
+static bool combos_ok(View X, int64_t r_blk, int64_t c_blk, int es = 2) {
+    const int epc = 16 / es;
     if (!aligned_to(X.p, 16)) return false;
-    if (X.cs == 1) return c_blk % 8 == 0 && X.rs % 8 == 0;
-    if (X.rs == 1) return r_blk % 8 == 0 && X.cs % 8 == 0;
+    if (X.cs == 1) return c_blk % epc == 0 && X.rs % epc == 0;
+    if (X.rs == 1) return r_blk % epc == 0 && X.cs % epc == 0;
     return false;
 }
 
@@ -890,6 +915,52 @@ struct Term { int a, b, sign; };
 static const Term kATerms[7] = {{0, 3, +1}, {2, 3, +1}, {0, 0, 0}, {3, 0, 0}, {0, 1, +1}, {2, 0, -1}, {1, 3, -1}};
 static const Term kBTerms[7] = {{0, 3, +1}, {0, 0, 0}, {1, 3, -1}, {2, 0, -1}, {3, 0, 0}, {0, 1, +1}, {2, 3, +1}};
 
+// sums by product M1..M7 as indices into the outputs of kStrA / kStrB (-1 = a raw block)
+static const int kSumA[7] = {2, 1, -1, -1, 0, 4, 3};
+static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
+
+// fp32, one Strassen level on the 256 x 256 kernel: the ten quadrant sums in one launch, the
+// seven products (reference numbering M1..M7, raw quadrants read in place) as one grouped launch
+// into seven dense fp32 matrices, one recombination pass.  Nothing is rounded anywhere.
+static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
+                                 bool accumulate, char* ws, hipStream_t stream) {
+    const size_t sa = align256(Mh * Kh * 4), sb = align256(Kh * Nh * 4), sm = align256(Mh * Nh * 4);
+    char* SA = ws;
+    char* SB = SA + 5 * sa;
+    char* Mbuf = SB + 5 * sb;
+    ComboPair pp;
+    const int64_t na = fill_combo(pp.side[0], A, Mh, Kh, SA, sa, 5, kStrA, 4);
+    const int64_t nb = fill_combo(pp.side[1], B, Kh, Nh, SB, sb, 5, kStrB, 4);
+    dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+    if (g_stages & 1) {
+        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos (fp32)");
+        if (rc) return rc;
+    }
+    const bool b_kc = B.rs == 1;
+    Gemm2Params g;
+    memset(&g, 0, sizeof(g));
+    for (int q = 0; q < 7; ++q) {
+        const Term ta = kATerms[q], tb = kBTerms[q];
+        const char* a = kSumA[q] < 0 ? A.p + ((int64_t)(ta.a >> 1) * Mh * A.rs + (int64_t)(ta.a & 1) * Kh) * 4 : SA + (size_t)kSumA[q] * sa;
+        const int64_t a_ld = kSumA[q] < 0 ? A.rs : Kh;
+        const char* b = kSumB[q] < 0 ? B.p + ((int64_t)(tb.a >> 1) * Kh * B.rs + (int64_t)(tb.a & 1) * Nh * B.cs) * 4 : SB + (size_t)kSumB[q] * sb;
+        const int64_t b_ld = kSumB[q] < 0 ? (b_kc ? B.cs : B.rs) : (b_kc ? Kh : Nh);   // sums keep B's storage orientation
+        g.seg[q] = Seg2{a, b, a_ld, b_ld, 0, 0};
+    }
+    g.C = Mbuf; g.c_rs = Nh; g.c_ps = (int64_t)(sm / 4); g.c_bs = 0;
+    g.Mh = (int)Mh; g.Nh = (int)Nh; g.Kh = (int)Kh;
+    g.tiles_m = (int)(Mh / kBM4); g.tiles_n = (int)(Nh / kBN4);
+    g.out_f32 = 1; g.accumulate = 0; g.group_m = 4; g.nprod = 7;
+    if (g_stages & 2) {
+        hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, stream);
+        if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    }
+    if (!(g_stages & 4)) return STHIP_OK;
+    return recombine(STHIP_F32, C, c_rs, 1, reinterpret_cast<const float*>(Mbuf), (int64_t)(sm / 4), Mh, Nh, 2 * Mh, 2 * Nh,
+                     accumulate, stream);
+}
+
 static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels) {
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
     if (levels <= 0) return 0;
@@ -931,9 +1002,9 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1) && ws && aligned_to(ws, 256) &&
         ws_bytes >= two_level_bytes(mh, nh, kh))
         return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, stream);
-    // Whole, aligned 16-bit problems: all five sums of each operand in one bandwidth-bound launch.
+    // Whole, aligned problems: all five sums of each operand in one bandwidth-bound launch.
     const bool whole = M == Mp && N == Np && K == Kp;
-    const bool vec = dt != STHIP_F32 && whole && combos_ok(A, mh, kh) && combos_ok(B, kh, nh);
+    const bool vec = whole && combos_ok(A, mh, kh, (int)es) && combos_ok(B, kh, nh, (int)es);
     const size_t sa_b = align256(mh * kh * es), sb_b = align256(kh * nh * es);
     const size_t m_b = align256(mh * nh * 4);
     const size_t need = 5 * (sa_b + sb_b) + 7 * m_b;
@@ -944,15 +1015,20 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     char* child_ws = ws + need;
     const size_t child_bytes = ws_bytes - need;
 
-    if (vec) {
+    if (vec && dt == STHIP_F32) {
+        ComboPair pp;
+        const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA, sa_b, 5, kStrA, 4);
+        const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB, sb_b, 5, kStrB, 4);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos (fp32)");
+        if (rc) return rc;
+    } else if (vec) {
         int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, stream);
         if (rc) return rc;
         rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, stream);
         if (rc) return rc;
     }
-    // sums by product M1..M7 as indices into the outputs of kStrA / kStrB (-1 = a raw block)
-    static const int kSumA[7] = {2, 1, -1, -1, 0, 4, 3};
-    static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
 
     for (int q = 0; q < 7; ++q) {
         const Term ta = kATerms[q], tb = kBTerms[q];

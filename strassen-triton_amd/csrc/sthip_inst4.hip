@@ -1,10 +1,12 @@
-// Instantiates the 256 x 256 pipelined grouped-GEMM kernel for one 16-bit element type:
-// -DSTHIP_INST_TYPE={1:f16,2:bf16}.
+// Instantiates the 256 x 256 pipelined grouped-GEMM kernel for one element type:
+// -DSTHIP_INST_TYPE={0:f32,1:f16,2:bf16}.
 #include "sthip_launch.hpp"
 
 namespace sthip {
 
-#if STHIP_INST_TYPE == 1
+#if STHIP_INST_TYPE == 0
+typedef float InstT;
+#elif STHIP_INST_TYPE == 1
 typedef f16_t InstT;
 #else
 typedef bf16_t InstT;

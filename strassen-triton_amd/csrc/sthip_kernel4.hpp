@@ -29,7 +29,10 @@
 namespace sthip {
 
 constexpr int kThreads4 = 256;
-constexpr int kBM4 = 256, kBN4 = 256, kBK4 = 64;
+constexpr int kBM4 = 256, kBN4 = 256, kBK4 = 64;   // kBK4: 16-bit elements per k-step (128 bytes per row)
+constexpr int kRowBytes4 = 128;                     // bytes of one tile row along k, any element type
+template <class T> constexpr int es4() { return __is_same(T, float) ? 4 : 2; }     // element size
+template <class T> constexpr int bk4() { return kRowBytes4 / es4<T>(); }           // elements per k-step
 constexpr int kStages4 = 2;
 constexpr int kATile4 = kBM4 * kBK4 * 2;                 // 32 KiB
 constexpr int kBTile4 = kBN4 * kBK4 * 2;                 // 32 KiB
@@ -39,7 +42,11 @@ constexpr int kSmemBytes4 = kStages4 * kStageBytes4;     // 128 KiB
 // A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 64 w + 8 i + L/8, i = 0..7,
 // chunk (L%8) ^ ((row/2)%8).  n-contiguous B: 64 k-rows x 32 chunks (512 bytes); wave w loads
 // k-rows 16 w + 2 i + L/32, i = 0..7, chunk (L%32) ^ ((k%4)*4) ^ (((k/8)%2)*2).
-template <bool B_KC>
+// fp32 operands use the same bytes: a k-step is 32 elements, a 16-byte chunk four of them.  The
+// n-contiguous fp32 B tile is 32 k-rows x 1024 bytes, one row per load: wave w loads k-rows
+// 8 w + i, and slot s of row k holds chunk s ^ (((k / 4) % 4) * 4), so that the four k-rows a
+// fragment read touches (k = 4 g + c, lane group g) fall into different 64-byte bank groups.
+template <int ES, bool B_KC>
 struct Loader4 {
     const char* a_base; const char* b_base;
     int64_t a_row_bytes, b_row_bytes, a_step_bytes, b_step_bytes;
@@ -51,20 +58,28 @@ struct Loader4 {
     __device__ __forceinline__ void point_at_segment() {
         const Seg2& s = P->seg[seg];
         const int lane = threadIdx.x & 63;
-        const char* a = reinterpret_cast<const char*>(s.a) + (int64_t)batch * s.a_bs * 2;
-        const char* b = reinterpret_cast<const char*>(s.b) + (int64_t)batch * s.b_bs * 2;
+        const char* a = reinterpret_cast<const char*>(s.a) + (int64_t)batch * s.a_bs * ES;
+        const char* b = reinterpret_cast<const char*>(s.b) + (int64_t)batch * s.b_bs * ES;
         const int chunk0 = (lane & 7) ^ (lane >> 4);     // (row/2)%8 = 4 (i%2) + L/16
-        a_base = a + (int64_t)(tile_m + wave * 64) * s.a_ld * 2;
-        a_row_bytes = 8 * s.a_ld * 2;
-        a_step_bytes = kBK4 * 2;
-        a_voff[0] = (uint32_t)(((lane >> 3) * s.a_ld + chunk0 * 8) * 2);
-        a_voff[1] = (uint32_t)(((lane >> 3) * s.a_ld + (chunk0 ^ 4) * 8) * 2);
+        a_base = a + (int64_t)(tile_m + wave * 64) * s.a_ld * ES;
+        a_row_bytes = 8 * s.a_ld * ES;
+        a_step_bytes = kRowBytes4;
+        a_voff[0] = (uint32_t)((lane >> 3) * s.a_ld * ES + chunk0 * 16);
+        a_voff[1] = (uint32_t)((lane >> 3) * s.a_ld * ES + (chunk0 ^ 4) * 16);
         if constexpr (B_KC) {
-            b_base = b + (int64_t)(tile_n + wave * 64) * s.b_ld * 2;
-            b_row_bytes = 8 * s.b_ld * 2;
-            b_step_bytes = kBK4 * 2;
-            b_voff[0] = b_voff[2] = (uint32_t)(((lane >> 3) * s.b_ld + chunk0 * 8) * 2);
-            b_voff[1] = b_voff[3] = (uint32_t)(((lane >> 3) * s.b_ld + (chunk0 ^ 4) * 8) * 2);
+            b_base = b + (int64_t)(tile_n + wave * 64) * s.b_ld * ES;
+            b_row_bytes = 8 * s.b_ld * ES;
+            b_step_bytes = kRowBytes4;
+            b_voff[0] = b_voff[2] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
+            b_voff[1] = b_voff[3] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
+        } else if constexpr (ES == 4) {
+            // k-row of load i: k = 8 w + i, so (k/4)%4 = (2 w + i/4) % 4
+            b_base = b + ((int64_t)(wave * 8) * s.b_ld + tile_n) * 4;
+            b_row_bytes = s.b_ld * 4;
+            b_step_bytes = (int64_t)kRowBytes4 * s.b_ld;
+#pragma unroll
+            for (int v = 0; v < 2; ++v)
+                b_voff[v] = b_voff[v + 2] = (uint32_t)((lane ^ (((2 * wave + v) & 3) << 2)) * 16);
         } else {
             // k-row of load i: k = 16 w + 2 i + L/32, so k%4 = 2 (i%2) + L/32 and (k/8)%2 = i/4;
             // the chunk stored in slot s of row k is s ^ ((k%4) * 4) ^ (((k/8)%2) * 2)
@@ -78,13 +93,19 @@ struct Loader4 {
         }
     }
 
+    // which b_voff the wave's load i of the B tile uses
+    static __device__ __forceinline__ int bv(int i) {
+        if constexpr (!B_KC && ES == 4) return i >> 2;
+        else return (i & 1) | ((i >> 2) << 1);
+    }
+
     // The sixteen loads of one k-step (8 for A, 8 for B), then move the cursor on.
     __device__ __forceinline__ void issue(uint32_t stage_addr) {
         const uint32_t sa = stage_addr + wave * 8192, sb = stage_addr + kATile4 + wave * 8192;
 #pragma unroll
         for (int i = 0; i < 8; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[(i & 1) | ((i >> 2) << 1)], sb + i * 1024);
+        for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[bv(i)], sb + i * 1024);
         advance();
     }
 
@@ -93,7 +114,7 @@ struct Loader4 {
         if (q < 8) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], stage_addr + wave * 8192 + q * 1024);
         else {
             const int i = q - 8;
-            lds_dma16(b_base + i * b_row_bytes, b_voff[(i & 1) | ((i >> 2) << 1)], stage_addr + kATile4 + wave * 8192 + i * 1024);
+            lds_dma16(b_base + i * b_row_bytes, b_voff[bv(i)], stage_addr + kATile4 + wave * 8192 + i * 1024);
         }
     }
     __device__ __forceinline__ void advance() {
@@ -143,10 +164,27 @@ __device__ __forceinline__ u32x4 read_frag16_mc(const char* tile, int sub, int k
     return r;
 }
 
+// n-contiguous fp32 B tile (32 k-rows of 1024 bytes): component c of the fragment is the element
+// at k = 16 kg + 4 g + c (g = lane / 16), column sub + lane % 16 -- the same k a lane's 16-byte
+// read of a k-contiguous tile puts into component c.
+__device__ __forceinline__ u32x4 read_frag16_mc_f32(const char* tile, int sub, int kg) {
+    const int lane = threadIdx.x & 63;
+    const int e = sub + (lane & 15), g = lane >> 4;
+    const char* p = tile + (kg * 16 + g * 4) * 1024 + (((e >> 2) ^ (g << 2)) * 16) + (e & 3) * 4;
+    u32x4 r;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) r[c] = *reinterpret_cast<const uint32_t*>(p + c * 1024);
+    return r;
+}
+
 // acc (16 n x 16 m, transposed so that a lane holds four consecutive n) += B-fragment x A-fragment.
 // Written as assembly so that the accumulator is updated in place: given the builtin, the
 // register allocator puts result and addend in different registers and permutes the 64
 // accumulators back with ~180 register copies per k-step.
+// fp32: one v_mfma_f32_16x16x4 on component c of both fragments (k = 4 g + c for lane group g).
+__device__ __forceinline__ void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b) {
+    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
 template <class T>
 __device__ __forceinline__ void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b) {
     if constexpr (__is_same(T, bf16_t))
@@ -169,7 +207,7 @@ struct Acc4 {   // one 128 x 128 wave tile = 8 x 8 MFMA tiles = 256 registers
 
 template <class T, bool B_KC>
 struct Pipe4 {
-    Loader4<B_KC> ld;
+    Loader4<es4<T>(), B_KC> ld;
     char* smem;
     uint32_t smem_addr;
     int g, total, slot;
@@ -180,6 +218,7 @@ struct Pipe4 {
     __device__ __forceinline__ void read_pair(int buf, int sl, int kg, int r) {
         const char* s = smem + sl * kStageBytes4;
         if constexpr (B_KC) fb[buf][r] = read_frag16_kc(s + kATile4, wn + r * 16, kg);
+        else if constexpr (es4<T>() == 4) fb[buf][r] = read_frag16_mc_f32(s + kATile4, wn + r * 16, kg);
         else fb[buf][r] = read_frag16_mc(s + kATile4, wn + r * 16, kg);
         fa[buf][r] = read_frag16_kc(s, wm + r * 16, kg);
     }
@@ -238,10 +277,20 @@ struct Pipe4 {
                     if (!(STHIP_DBG & 4)) {
                         read_pair(nb, nsl, nkg, i);
                     }
+                    if constexpr (es4<T>() == 4) {
+                        // four matrix instructions per accumulator and k-group: component-major, so
+                        // that instructions on one accumulator are eight apart
 #pragma unroll
-                    for (int jj = 0; jj < 8; ++jj) {
-                        const int j = (i & 1) ? 7 - jj : jj;   // boustrophedon: the B fragment carries over between rows
-                        if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
+                        for (int c = 0; c < 4; ++c)
+#pragma unroll
+                            for (int j = 0; j < 8; ++j)
+                                if (!(STHIP_DBG & 64)) mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
+                    } else {
+#pragma unroll
+                        for (int jj = 0; jj < 8; ++jj) {
+                            const int j = (i & 1) ? 7 - jj : jj;   // boustrophedon: the B fragment carries over between rows
+                            if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -348,7 +397,7 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     const int batch = blockIdx.y;
     char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int KT = P.Kh / kBK4;
+    const int KT = P.Kh / bk4<T>();
 
     Pipe4<T, B_KC> pipe;
     pipe.smem = smem;

@@ -89,8 +89,9 @@ hipError_t launch_gemm3(const Gemm2Params& p, int batch, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// 256 x 256 kernel (16-bit operands, A contiguous along k), p.nprod products per launch:
+// 256 x 256 kernel (fp32 or 16-bit operands, A contiguous along k), p.nprod products per launch:
 // tables indexed [b_kc].
+extern const LaunchTable3 kLaunch4_0;
 extern const LaunchTable3 kLaunch4_1;
 extern const LaunchTable3 kLaunch4_2;
 

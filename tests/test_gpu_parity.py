@@ -396,3 +396,39 @@ def test_large_tile_store_alignment(hip, monkeypatch, dtype, pad, off, algo, lev
     hip.gemm(A.cuda(), B.cuda(), out=out, algo=algo, levels=levels)
     assert torch.equal(out.cpu().double(), want)
     assert torch.all(buf[:, :off] == 7) and torch.all(buf[:, off + N:] == 7)
+
+
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("algo,levels,shape,batch", [
+    ("classic", 0, (4096, 4096, 96), 1),       # 256 tiles of 256 x 256
+    ("classic", 0, (2048, 2048, 64), 4),       # the batch fills the chip
+    ("strassen", 1, (4096, 2048, 128), 1),     # seven grouped products of 2048 x 1024 x 64
+    ("strassen", 2, (8192, 4096, 256), 1),     # the children of the host recursion take the same path
+])
+def test_fp32_large_tile_exact(hip, algo, levels, shape, batch, tb):
+    """fp32 problems with enough 256 x 256 tiles run on the pipelined kernel (classical directly,
+    one Strassen level as sums + one grouped launch + recombination): exact on small integers, both
+    B layouts, plain and accumulating."""
+    M, N, K = shape
+    A, B = _ints((batch, M, K), 71, -2, 2), _ints((batch, K, N), 72, -2, 2)
+    want = A.double() @ B.double()
+    Bg = _layout(B, tb)
+    if batch == 1:
+        A, Bg, want = A[0], Bg[0], want[0]
+    C = hip.gemm(A.cuda(), Bg, algo=algo, levels=levels)
+    assert C.dtype == torch.float32 and torch.equal(C.cpu().double(), want)
+    C0 = _ints(tuple(want.shape), 73, -3, 3)
+    Cacc = C0.clone().cuda()
+    hip.gemm(A.cuda(), Bg, out=Cacc, algo=algo, levels=levels, accumulate=True)
+    assert torch.equal(Cacc.cpu().double(), C0.double() + want)
+
+
+def test_fp32_large_tile_gaussian(hip):
+    """Seeded Gaussian 4096^3 fp32, one Strassen level on the pipelined kernel, against fp64."""
+    n = 4096
+    A, B = _gauss((n, n), 81, 1.0, torch.float32), _gauss((n, n), 82, 1.0, torch.float32)
+    want = A.double() @ B.double()
+    C = hip.gemm(A.cuda(), B.cuda(), algo="strassen", levels=1).cpu().double()
+    err = float(torch.linalg.norm(C - want) / torch.linalg.norm(want))
+    print(f"fp32 4096^3 one level: rel_fro vs fp64 {err:.3e}")
+    assert err <= TOL[torch.float32]
