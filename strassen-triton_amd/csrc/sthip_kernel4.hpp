@@ -1,10 +1,10 @@
-// 256 x 256-tile pipelined grouped-GEMM kernel for gfx950: four waves (one per SIMD) of
-// 128 x 128 each, 16-bit operands, A contiguous along k.
+// 256 x 256-tile pipelined grouped-GEMM kernel for gfx950: eight waves (two per SIMD) of
+// 128 x 64 each, 16-bit or fp32 operands, A contiguous along k.
 //
 // The L2 -> LDS path, not the matrix cores, limits the smaller-tile kernels: bytes moved per
 // flop go with (1/BM + 1/BN).  A 256 x 256 tile moves two thirds of what 256 x 128 moves, but
-// one fp32 accumulator tile then fills all 256 AGPRs of a wave, so no Strassen / Winograd chain
-// can stay in registers beside it.  (Parking the chains in per-workgroup fp32 slabs was built
+// its fp32 accumulators then fill half of the CU's registers, so no Strassen / Winograd chain
+// can stay in registers beside them.  (Parking the chains in per-workgroup fp32 slabs was built
 // and measured: every CU parks 256 KiB at the same moment, nine to eighteen times per tile,
 // and the kernel ran a third slower than the 256 x 128 one.)  So this kernel only ever runs
 // plain products: one launch covers `nprod` independent products of equal shape (the seven
@@ -12,7 +12,14 @@
 // so that the chip works through one product at a time and each behaves like a classical GEMM.
 // The recombination of the seven outputs is a separate elementwise pass.
 //
-// Matrix instruction: v_mfma_f32_16x16x32 (a 128 x 128 wave tile is 8 x 8 of them per 32 k).
+// Two waves per SIMD, not one with a 128 x 128 tile: a wave issues in order, and with a single
+// wave per SIMD every LDS read and every direct-to-LDS load was measured to cost its own issue
+// time on top of the matrix instructions (the costs added up instead of overlapping); the second
+// wave fills those gaps (+3.5 % at 8192^3 bf16, +2.5 % fp32) at the price of half as many more
+// fragment reads.
+//
+// Matrix instruction: v_mfma_f32_16x16x32 (a 128 x 64 wave tile is 8 x 4 of them per 32 k); fp32
+// operands: v_mfma_f32_16x16x4_f32, four per 16-byte fragment pair.
 // Sustained matrix throughput on this card is set by the power limit, and with random operands
 // the 16x16x32 form sustains 14 % more than 32x32x16 in a register-only loop (2.08 against 1.82
 // PFLOP/s); in this kernel it is worth 1 - 4 %.
@@ -28,7 +35,7 @@
 
 namespace sthip {
 
-constexpr int kThreads4 = 256;
+constexpr int kThreads4 = 512;   // eight waves, two per SIMD
 constexpr int kBM4 = 256, kBN4 = 256, kBK4 = 64;   // kBK4: 16-bit elements per k-step (128 bytes per row)
 constexpr int kRowBytes4 = 128;                     // bytes of one tile row along k, any element type
 template <class T> constexpr int es4() { return __is_same(T, float) ? 4 : 2; }     // element size
@@ -39,18 +46,18 @@ constexpr int kBTile4 = kBN4 * kBK4 * 2;                 // 32 KiB
 constexpr int kStageBytes4 = kATile4 + kBTile4;          // 64 KiB
 constexpr int kSmemBytes4 = kStages4 * kStageBytes4;     // 128 KiB
 
-// A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 64 w + 8 i + L/8, i = 0..7,
+// A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 32 w + 8 i + L/8, i = 0..3,
 // chunk (L%8) ^ ((row/2)%8).  n-contiguous B: 64 k-rows x 32 chunks (512 bytes); wave w loads
-// k-rows 16 w + 2 i + L/32, i = 0..7, chunk (L%32) ^ ((k%4)*4) ^ (((k/8)%2)*2).
+// k-rows 8 w + 2 i + L/32, i = 0..3, chunk (L%32) ^ ((k%4)*4) ^ (((k/8)%2)*2).
 // fp32 operands use the same bytes: a k-step is 32 elements, a 16-byte chunk four of them.  The
 // n-contiguous fp32 B tile is 32 k-rows x 1024 bytes, one row per load: wave w loads k-rows
-// 8 w + i, and slot s of row k holds chunk s ^ (((k / 4) % 4) * 4), so that the four k-rows a
+// 4 w + i (i = 0..3), and slot s of row k holds chunk s ^ (((k / 4) % 4) * 4), so that the four k-rows a
 // fragment read touches (k = 4 g + c, lane group g) fall into different 64-byte bank groups.
 template <int ES, bool B_KC>
 struct Loader4 {
     const char* a_base; const char* b_base;
     int64_t a_row_bytes, b_row_bytes, a_step_bytes, b_step_bytes;
-    uint32_t a_voff[2], b_voff[4];   // b: index (i % 2) + 2 (i / 4) of the wave's load i
+    uint32_t a_voff[2], b_voff[2];   // index i % 2 of the wave's load i
     int seg, kt, total_seg, KT;
     int batch, tile_m, tile_n, wave;
     const Gemm2Params* P;
@@ -61,60 +68,52 @@ struct Loader4 {
         const char* a = reinterpret_cast<const char*>(s.a) + (int64_t)batch * s.a_bs * ES;
         const char* b = reinterpret_cast<const char*>(s.b) + (int64_t)batch * s.b_bs * ES;
         const int chunk0 = (lane & 7) ^ (lane >> 4);     // (row/2)%8 = 4 (i%2) + L/16
-        a_base = a + (int64_t)(tile_m + wave * 64) * s.a_ld * ES;
+        a_base = a + (int64_t)(tile_m + wave * 32) * s.a_ld * ES;
         a_row_bytes = 8 * s.a_ld * ES;
         a_step_bytes = kRowBytes4;
         a_voff[0] = (uint32_t)((lane >> 3) * s.a_ld * ES + chunk0 * 16);
         a_voff[1] = (uint32_t)((lane >> 3) * s.a_ld * ES + (chunk0 ^ 4) * 16);
         if constexpr (B_KC) {
-            b_base = b + (int64_t)(tile_n + wave * 64) * s.b_ld * ES;
+            b_base = b + (int64_t)(tile_n + wave * 32) * s.b_ld * ES;
             b_row_bytes = 8 * s.b_ld * ES;
             b_step_bytes = kRowBytes4;
-            b_voff[0] = b_voff[2] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
-            b_voff[1] = b_voff[3] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
+            b_voff[0] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
+            b_voff[1] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
         } else if constexpr (ES == 4) {
-            // k-row of load i: k = 8 w + i, so (k/4)%4 = (2 w + i/4) % 4
-            b_base = b + ((int64_t)(wave * 8) * s.b_ld + tile_n) * 4;
+            // k-row of load i: k = 4 w + i, so (k/4)%4 = w % 4
+            b_base = b + ((int64_t)(wave * 4) * s.b_ld + tile_n) * 4;
             b_row_bytes = s.b_ld * 4;
             b_step_bytes = (int64_t)kRowBytes4 * s.b_ld;
-#pragma unroll
-            for (int v = 0; v < 2; ++v)
-                b_voff[v] = b_voff[v + 2] = (uint32_t)((lane ^ (((2 * wave + v) & 3) << 2)) * 16);
+            b_voff[0] = b_voff[1] = (uint32_t)((lane ^ ((wave & 3) << 2)) * 16);
         } else {
-            // k-row of load i: k = 16 w + 2 i + L/32, so k%4 = 2 (i%2) + L/32 and (k/8)%2 = i/4;
+            // k-row of load i: k = 8 w + 2 i + L/32, so k%4 = 2 (i%2) + L/32 and (k/8)%2 = w%2;
             // the chunk stored in slot s of row k is s ^ ((k%4) * 4) ^ (((k/8)%2) * 2)
             const int chunk = (lane & 31) ^ ((lane >> 5) << 2);
-            b_base = b + ((int64_t)(wave * 16) * s.b_ld + tile_n) * 2;
+            b_base = b + ((int64_t)(wave * 8) * s.b_ld + tile_n) * 2;
             b_row_bytes = 2 * s.b_ld * 2;
             b_step_bytes = (int64_t)kBK4 * s.b_ld * 2;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                b_voff[v] = (uint32_t)(((lane >> 5) * s.b_ld + (chunk ^ ((v & 1) << 3) ^ ((v >> 1) << 1)) * 8) * 2);
+            for (int v = 0; v < 2; ++v)
+                b_voff[v] = (uint32_t)(((lane >> 5) * s.b_ld + (chunk ^ (v << 3) ^ ((wave & 1) << 1)) * 8) * 2);
         }
     }
 
-    // which b_voff the wave's load i of the B tile uses
-    static __device__ __forceinline__ int bv(int i) {
-        if constexpr (!B_KC && ES == 4) return i >> 2;
-        else return (i & 1) | ((i >> 2) << 1);
-    }
-
-    // The sixteen loads of one k-step (8 for A, 8 for B), then move the cursor on.
+    // The wave's eight loads of one k-step (4 for A, 4 for B), then move the cursor on.
     __device__ __forceinline__ void issue(uint32_t stage_addr) {
-        const uint32_t sa = stage_addr + wave * 8192, sb = stage_addr + kATile4 + wave * 8192;
+        const uint32_t sa = stage_addr + wave * 4096, sb = stage_addr + kATile4 + wave * 4096;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
+        for (int i = 0; i < 4; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[bv(i)], sb + i * 1024);
+        for (int i = 0; i < 4; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], sb + i * 1024);
         advance();
     }
 
-    // Load q (0..7 the A tile, 8..15 the B tile) of the next k-step; advance() after the sixteenth.
+    // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step; advance() after the eighth.
     __device__ __forceinline__ void issue_one(uint32_t stage_addr, int q) {
-        if (q < 8) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], stage_addr + wave * 8192 + q * 1024);
+        if (q < 4) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], stage_addr + wave * 4096 + q * 1024);
         else {
-            const int i = q - 8;
-            lds_dma16(b_base + i * b_row_bytes, b_voff[bv(i)], stage_addr + kATile4 + wave * 8192 + i * 1024);
+            const int i = q - 4;
+            lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], stage_addr + kATile4 + wave * 4096 + i * 1024);
         }
     }
     __device__ __forceinline__ void advance() {
@@ -193,13 +192,13 @@ __device__ __forceinline__ void mfma16_step(f32x4& acc, const u32x4& a, const u3
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
 }
 
-struct Acc4 {   // one 128 x 128 wave tile = 8 x 8 MFMA tiles = 256 registers
-    f32x4 t[8][8];
+struct Acc4 {   // one 128 x 64 wave tile = 8 x 4 MFMA tiles = 128 registers
+    f32x4 t[8][4];
     __device__ __forceinline__ void zero() {
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) t[i][j][e] = 0.f;
     }
@@ -212,14 +211,16 @@ struct Pipe4 {
     uint32_t smem_addr;
     int g, total, slot;
     int wm, wn;
-    u32x4 fa[2][8], fb[2][8];   // [buffer][16-wide block]: fragments of one group of 32 k
+    u32x4 fa[2][8], fb[2][4];   // [buffer][16-wide block]: fragments of one group of 32 k
 
-    // The A and the B fragment of 16-wide block r.
+    // The A fragment of 16-wide block r and, for r < 4, the B fragment.
     __device__ __forceinline__ void read_pair(int buf, int sl, int kg, int r) {
         const char* s = smem + sl * kStageBytes4;
-        if constexpr (B_KC) fb[buf][r] = read_frag16_kc(s + kATile4, wn + r * 16, kg);
-        else if constexpr (es4<T>() == 4) fb[buf][r] = read_frag16_mc_f32(s + kATile4, wn + r * 16, kg);
-        else fb[buf][r] = read_frag16_mc(s + kATile4, wn + r * 16, kg);
+        if (r < 4) {
+            if constexpr (B_KC) fb[buf][r] = read_frag16_kc(s + kATile4, wn + r * 16, kg);
+            else if constexpr (es4<T>() == 4) fb[buf][r] = read_frag16_mc_f32(s + kATile4, wn + r * 16, kg);
+            else fb[buf][r] = read_frag16_mc(s + kATile4, wn + r * 16, kg);
+        }
         fa[buf][r] = read_frag16_kc(s, wm + r * 16, kg);
     }
     __device__ __forceinline__ void read_frags(int buf, int sl, int kg) {
@@ -234,12 +235,12 @@ struct Pipe4 {
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i] = u32x4{0, 0, 0, 0}; }
+                for (int i = 0; i < 8; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i & 3] = u32x4{0, 0, 0, 0}; }
         }
         if (!(STHIP_DBG & 1)) {
             ld.issue(smem_addr);
             if (!ld.done()) ld.issue(smem_addr + kStageBytes4);
-            if (total >= 2) wait_vmcnt_imm<16>(); else wait_vmcnt_imm<0>();   // step 0 has landed
+            if (total >= 2) wait_vmcnt_imm<8>(); else wait_vmcnt_imm<0>();   // step 0 has landed
         }
         __syncthreads();
         if (!(STHIP_DBG & 4)) read_frags(0, 0, 0);
@@ -257,38 +258,36 @@ struct Pipe4 {
                     if (!(STHIP_DBG & 1)) wait_vmcnt_imm<0>();
                     if (!(STHIP_DBG & 2)) __syncthreads();
                 }
-                // The sixteen loads of step g+2 go out four per row over the first four rows of matrix
-                // instructions (measured at 8192^3: all sixteen at once 0.953 ms, eight per row 0.925,
-                // four 0.900, two 0.917).
+                // The wave's eight loads of step g+2 go out one per row of matrix instructions
+                // (measured at 8192^3: one per row 0.865 ms, two 0.879, four or all at once 0.895).
                 const bool issuing = kg == 1 && !(STHIP_DBG & 1) && !ld.done();
                 // Fragments of the next k-group come in between the rows of matrix instructions, one
-                // A and one B fragment (two or three LDS reads) per row: few enough in flight for the
-                // LDS counter (4 bits) to tell the old fragments from the new -- with all 24 reads
-                // issued first, the first matrix instruction waited for ten of them.  In the last
-                // step the "next" fragments are stale data that nobody uses.
+                // A and (first four rows) one B fragment per row: few enough in flight for the LDS
+                // counter (4 bits) to tell the old fragments from the new, and bursts of reads cost
+                // more (two pairs per row 0.878 ms, all up front 0.900).  In the last step the
+                // "next" fragments are stale data that nobody uses.
                 const int nsl = kg == 0 ? slot : slot ^ 1, nkg = kg ^ 1;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    if (issuing && i < 4) {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) ld.issue_one(smem_addr + slot * kStageBytes4, 4 * i + q);
-                        if (i == 3) ld.advance();
+                    if (issuing) {
+                        ld.issue_one(smem_addr + slot * kStageBytes4, i);
+                        if (i == 7) ld.advance();
                     }
                     if (!(STHIP_DBG & 4)) {
                         read_pair(nb, nsl, nkg, i);
                     }
                     if constexpr (es4<T>() == 4) {
                         // four matrix instructions per accumulator and k-group: component-major, so
-                        // that instructions on one accumulator are eight apart
+                        // that instructions on one accumulator are four apart
 #pragma unroll
                         for (int c = 0; c < 4; ++c)
 #pragma unroll
-                            for (int j = 0; j < 8; ++j)
+                            for (int j = 0; j < 4; ++j)
                                 if (!(STHIP_DBG & 64)) mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
                     } else {
 #pragma unroll
-                        for (int jj = 0; jj < 8; ++jj) {
-                            const int j = (i & 1) ? 7 - jj : jj;   // boustrophedon: the B fragment carries over between rows
+                        for (int jj = 0; jj < 4; ++jj) {
+                            const int j = (i & 1) ? 3 - jj : jj;   // boustrophedon: the B fragment carries over between rows
                             if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                         }
                     }
@@ -313,7 +312,7 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 4; ++j) {
             float v[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc.t[i][j][e];
@@ -346,10 +345,10 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
 }
 
 // The 16-bit, non-accumulating store, staged through LDS so that every store instruction writes
-// four rows x 256 contiguous bytes (16 bytes per lane) instead of sixteen rows x 32 bytes: with
+// eight rows x 128 contiguous bytes (16 bytes per lane) instead of sixteen rows x 32 bytes: with
 // all workgroups of a round storing at once, the partial-line pattern of the MFMA layout costs
-// about twice the time.  Each wave uses its own 32 KiB of the (now idle) stage buffers: row r of
-// its 128 x 128 tile at r * 256, the 8-byte chunk c of a row at ((c ^ 2 (r % 16)) * 8, which
+// about twice the time.  Each wave uses its own 16 KiB of the (now idle) stage buffers: row r of
+// its 128 x 64 tile at r * 128, the 8-byte chunk c of a row at (c ^ 2 ((r / 2) % 8)) * 8, which
 // spreads the sixteen rows a write instruction touches over all banks and keeps 16-byte chunks
 // whole for the read back.  The caller has synchronised the workgroup.
 template <class T>
@@ -357,27 +356,28 @@ __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Para
                                                 int wave, int row, int col) {
     const int lane = threadIdx.x & 63;
     const int l16 = lane & 15, q = lane >> 4;
-    char* w = smem + wave * 32768;
-    uint32_t waddr[8];
+    char* w = smem + wave * 16384;
+    uint32_t waddr[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) waddr[j] = l16 * 256 + (((4 * j + q) ^ (2 * l16)) * 8);
+    for (int j = 0; j < 4; ++j) waddr[j] = l16 * 128 + (((4 * j + q) ^ (2 * (l16 >> 1))) * 8);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 4; ++j) {
             u32x2 o;
             if constexpr (__is_same(T, bf16_t)) { o[0] = pack_bf16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_bf16(acc.t[i][j][2], acc.t[i][j][3]); }
             else { o[0] = pack_f16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_f16(acc.t[i][j][2], acc.t[i][j][3]); }
-            *reinterpret_cast<u32x2*>(w + i * 4096 + waddr[j]) = o;
+            *reinterpret_cast<u32x2*>(w + i * 2048 + waddr[j]) = o;
         }
     }
-    // read back: lane -> row 4 r + q, 16-byte chunk l16; the same wave wrote it, LDS keeps order
-    char* dst = Cb + ((int64_t)(row + q) * P.c_rs + (col + 8 * l16)) * 2;
-    const int64_t step = (int64_t)4 * P.c_rs * 2;
+    // read back: lane -> row 8 r + lane / 8, 16-byte chunk lane % 8; the same wave wrote it, LDS keeps order
+    const int r8 = lane >> 3, c16 = lane & 7;
+    char* dst = Cb + ((int64_t)(row + r8) * P.c_rs + (col + 8 * c16)) * 2;
+    const int64_t step = (int64_t)8 * P.c_rs * 2;
 #pragma unroll
-    for (int r = 0; r < 32; ++r) {
-        const int rr = 4 * (r & 3) + q;                       // (4 r + q) % 16
-        const u32x4 v = *reinterpret_cast<const u32x4*>(w + (4 * r + q) * 256 + ((l16 ^ rr) * 16));
+    for (int r = 0; r < 16; ++r) {
+        const int rr = ((8 * r + r8) >> 1) & 7;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(w + (8 * r + r8) * 128 + ((c16 ^ rr) * 16));
         *reinterpret_cast<u32x4*>(dst + r * step) = v;
     }
 }
@@ -402,8 +402,8 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     Pipe4<T, B_KC> pipe;
     pipe.smem = smem;
     pipe.smem_addr = (uint32_t)(uintptr_t)(lptr_t)smem;
-    pipe.wm = (wave >> 1) * 128;
-    pipe.wn = (wave & 1) * 128;
+    pipe.wm = (wave >> 2) * 128;
+    pipe.wn = (wave & 3) * 64;
     pipe.total = KT;
     pipe.ld.P = &P;
     pipe.ld.wave = wave;
