@@ -58,8 +58,10 @@ enum sthip_algo {
  * operand type) use 256 x 256 tiles, round each product once to the operand type as the
  * reference's mm does, and recombine in a third pass in fp32; the others recombine in
  * registers without that rounding.  fp32 problems with tile-aligned half-size blocks (128 x 128
- * x 32) and workspace run the seven products as one batched launch over dense operand copies;
- * nothing is rounded.  levels = 2 on tile-aligned 16-bit problems runs as five
+ * x 32) and workspace write their sums once and run the seven products as one launch (grouped on
+ * 256 x 256 tiles when A is contiguous along k and the blocks are multiples of 256 and large
+ * enough to fill the chip, else batched over dense operand copies); nothing is rounded.  Plain
+ * products (STHIP_CLASSIC) of all three types take the 256 x 256 kernel under the same conditions.  levels = 2 on tile-aligned 16-bit problems runs as five
  * launches (sums of both levels, ONE grouped GEMM of the 49 quarter-size products, two
  * recombination passes; every level returns its products in the operand type, the first level
  * is always Strassen).  Otherwise levels >= 2 recurses on
