@@ -56,8 +56,9 @@ enum sthip_algo {
  * pipelined path instead: the quadrant sums are written once, then one grouped-GEMM launch
  * runs the seven products.  Large problems (half-size blocks multiples of 256, result in the
  * operand type) use 256 x 256 tiles, round each product once to the operand type as the
- * reference's mm does, and recombine in a third pass in fp32; the others recombine in
- * registers without that rounding.  fp32 problems with tile-aligned half-size blocks (128 x 128
+ * reference's mm does, and recombine in a third pass in fp32; with an fp32 result the seven
+ * products are kept in fp32 instead (never rounded, as in the reference's Triton kernels; the
+ * workspace query then asks for twice the product room); the others recombine in registers.  fp32 problems with tile-aligned half-size blocks (128 x 128
  * x 32) and workspace write their sums once and run the seven products as one launch (grouped on
  * 256 x 256 tiles when A is contiguous along k and the blocks are multiples of 256 and large
  * enough to fill the chip, else batched over dense operand copies); nothing is rounded.  Plain

@@ -192,9 +192,10 @@ static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0,
 // Workspace of the pipelined path per problem: five sums per operand, then a region that is
 // either the seven 16-bit products of the 256 x 256 grouped launch or the fp32 slabs in which
 // the 256 x 128 kernel parks one accumulator tile per workgroup (at most Mh x Nh floats).
-static size_t products_bytes(int64_t Mh, int64_t Nh) { return 7 * align256(Mh * Nh * 2); }
-static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh) {
-    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + products_bytes(Mh, Nh));
+// (prod_es = 4: the seven products kept in fp32, for 16-bit operands with an fp32 result.)
+static size_t products_bytes(int64_t Mh, int64_t Nh, int prod_es = 2) { return 7 * align256(Mh * Nh * prod_es); }
+static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh, int prod_es = 2) {
+    return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + products_bytes(Mh, Nh, prod_es));
 }
 
 // Recombination of the seven 16-bit products of one level (kernel order: Strassen
@@ -274,6 +275,42 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
             else w[k] = pack_f16(out[q][2 * k], out[q][2 * k + 1]);
         }
         __builtin_nontemporal_store(w, d);
+    }
+}
+
+// The same recombination for seven fp32 products (16-bit operands, fp32 result: the products are
+// not rounded, as in the reference's Triton kernels, strassen.py:150-190): one thread per four
+// consecutive columns of a half-size row.
+template <int ALGO>
+__global__ void __launch_bounds__(256) recombine32_kernel(const Recombine16Params p) {
+    const int nq = p.Nh / 4;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.Mh * nq) return;
+    const int i = (int)(idx / nq), j = (int)(idx % nq) * 4;
+    const float* src = reinterpret_cast<const float*>(p.prod) + (int64_t)blockIdx.y * 7 * p.p_ps + (int64_t)i * p.Nh + j;
+    f32x4 m[7];
+#pragma unroll
+    for (int q = 0; q < 7; ++q) m[q] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + q * p.p_ps));
+    f32x4 out[4];
+    if constexpr (ALGO == STHIP_STRASSEN) {
+        out[0] = ((m[4] + m[6]) - m[2]) + m[3];   // C11 = M1 + M4 - M5 + M7
+        out[1] = m[0] + m[2];                     // C12 = M3 + M5
+        out[2] = m[5] + m[6];                     // C21 = M2 + M4
+        out[3] = ((m[4] - m[5]) + m[0]) + m[1];   // C22 = M1 - M2 + M3 + M6
+    } else {
+        const f32x4 u2 = m[0] + m[2], u3 = u2 + m[3], u4 = u2 + m[4];
+        out[0] = m[0] + m[1];                     // C11 = P1 + P2
+        out[1] = u4 + m[5];                       // C12 = U4 + P3
+        out[2] = u3 + m[6];                       // C21 = U3 - P4
+        out[3] = u3 + m[4];                       // C22 = U3 + P5
+    }
+    float* Cf = reinterpret_cast<float*>(p.C) + (int64_t)blockIdx.y * p.c_bs;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        f32x4* d = reinterpret_cast<f32x4*>(Cf + (int64_t)(i + (q >> 1) * p.Mh) * p.c_rs + (j + (q & 1) * p.Nh));
+        f32x4 v = out[q];
+        if (p.accumulate) v += *d;
+        *d = v;
     }
 }
 
@@ -378,10 +415,14 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     const LaunchTable3* t4 = table4_for(dt);
     const int force = forced_tile();
     const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
-    const bool grouped_ok = !split || (!out_f32 && c_vec);   // 16-bit products + recombination pass
+    // products as matrices + recombination pass: 16-bit products for a result in the operand type,
+    // fp32 products (twice the room) for an fp32 result
+    const bool f32_prod = split && out_f32 && c_rs % 4 == 0 && c_bs % 4 == 0 && aligned_to(C, 16) &&
+                          ws_bytes >= prepass_bytes(batch, Mh, Nh, Kh, 4);
+    const bool grouped_ok = !split || (out_f32 ? f32_prod : c_vec);
     const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && grouped_ok;
     const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
-    const bool can5 = split && grouped_ok;
+    const bool can5 = split && !out_f32 && grouped_ok;
     const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch * (split ? 7 : 1);
     const int64_t tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
     const int64_t tiles2 = (Mh / 128) * (Nh / 128) * batch;
@@ -402,10 +443,10 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     if ((pick == 4 || pick == 5) && split) {
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
-        rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0; rp.p_ps = Mh * Nh; rp.out_f32 = 0;
+        rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0; rp.p_ps = Mh * Nh; rp.out_f32 = out_f32 ? 1 : 0;
         if (g_stages & 2) {
             p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
-            p.out_f32 = 0; p.accumulate = 0; p.nprod = 7;
+            p.out_f32 = out_f32 ? 1 : 0; p.accumulate = 0; p.nprod = 7;
             if (pick == 4) {
                 p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
                 p.group_m = 4;
@@ -417,6 +458,12 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
                 e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
             }
             if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+        }
+        if ((g_stages & 4) && out_f32) {
+            dim3 grid((unsigned)ceil_div(Mh * (Nh / 4), 256), (unsigned)batch);
+            if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, stream, rp);
+            else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, stream, rp);
+            return check_launch("recombine32");
         }
         if (g_stages & 4) {
             dim3 grid((unsigned)ceil_div(Mh * (Nh / 8), 256), (unsigned)batch);
@@ -1114,7 +1161,6 @@ int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, 
 }
 
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {
-    (void)out_dtype;
     if (algo == STHIP_CLASSIC || levels <= 0 || M <= 0 || N <= 0 || K < 0 || levels > 8 || in_dtype < 0 || in_dtype > 2) return 0;
     const int64_t q = (int64_t)1 << levels;
     const int64_t Mp = round_up(M, q), Np = round_up(N, q), Kp = round_up(K, q);
@@ -1123,6 +1169,9 @@ size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int
     if (levels == 1) {
         if (Mp != M || Np != N || Kp != K) return 0;
         if (in_dtype == STHIP_F32) return batch == 1 ? workspace_for(Mp, Np, Kp, in_dtype, 1) : 0;   // batched-products path: one problem
+        // an fp32 result of 16-bit operands keeps its seven products in fp32
+        if (out_dtype == STHIP_F32 && fast_shape(in_dtype, Mp / 2, Np / 2, Kp / 2))
+            return prepass_bytes(batch, Mp / 2, Np / 2, Kp / 2, 4);
         return (size_t)batch * workspace_for(Mp, Np, Kp, in_dtype, 1);
     }
     return workspace_for(Mp, Np, Kp, in_dtype, levels);

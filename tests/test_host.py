@@ -64,6 +64,8 @@ def test_argument_errors_need_no_gpu():
     sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles)
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == sums(512)
     assert lib.sthip_workspace_bytes(3, 1024, 1024, 1024, 1, 1, 2, 1) == 3 * sums(512)
+    # 16-bit operands with an fp32 result: the seven products stay fp32
+    assert lib.sthip_workspace_bytes(2, 1024, 1024, 1024, 2, 0, 1, 1) == 2 * (2 * 5 * 512 * 512 * 2 + 7 * 512 * 512 * 4)
     # fp32, tile aligned: seven dense A operands, seven B operands, seven fp32 products
     f32 = lambda h: 7 * 3 * h * h * 4
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == f32(512)
