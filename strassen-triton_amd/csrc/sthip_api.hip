@@ -176,6 +176,7 @@ __global__ void __launch_bounds__(256) quad_combos_pair_f32_kernel(const ComboPa
 struct ComboMany { ComboParams side[14]; };
 template <class T>
 __global__ void __launch_bounds__(256) quad_combos_many_kernel(const ComboMany pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
+__global__ void __launch_bounds__(256) quad_combos_many_f32_kernel(const ComboMany pp) { quad_combos_f32_body(pp.side[blockIdx.z]); }
 
 // Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
 // Strassen (fixed_strassen.py:88-97): A side S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.
@@ -726,9 +727,9 @@ static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, s
 // quadrant is a view into the operand, a sum is dense in the operand's storage orientation at
 // S? + index * stride (index = output number of kStr? / kWin?).
 static void level_operands(int algo, View A, View B, int64_t mh, int64_t nh, int64_t kh,
-                           const char* SA, size_t sa_b, const char* SB, size_t sb_b, View xa[7], View xb[7]) {
-    auto rawA = [&](int q) { return View{A.p + ((int64_t)(q >> 1) * mh * A.rs + (int64_t)(q & 1) * kh * A.cs) * 2, A.rs, A.cs}; };
-    auto rawB = [&](int q) { return View{B.p + ((int64_t)(q >> 1) * kh * B.rs + (int64_t)(q & 1) * nh * B.cs) * 2, B.rs, B.cs}; };
+                           const char* SA, size_t sa_b, const char* SB, size_t sb_b, View xa[7], View xb[7], int es = 2) {
+    auto rawA = [&](int q) { return View{A.p + ((int64_t)(q >> 1) * mh * A.rs + (int64_t)(q & 1) * kh * A.cs) * es, A.rs, A.cs}; };
+    auto rawB = [&](int q) { return View{B.p + ((int64_t)(q >> 1) * kh * B.rs + (int64_t)(q & 1) * nh * B.cs) * es, B.rs, B.cs}; };
     auto sumA = [&](int o) { const char* p = SA + (size_t)o * sa_b; return A.cs == 1 ? View{p, kh, 1} : View{p, 1, mh}; };
     auto sumB = [&](int o) { const char* p = SB + (size_t)o * sb_b; return B.cs == 1 ? View{p, nh, 1} : View{p, 1, kh}; };
     if (algo == STHIP_STRASSEN) {
@@ -859,6 +860,89 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
     if (rc) return rc;
     return launch_recombine16(dt, STHIP_STRASSEN, Mp, (int64_t)(mb / 2), C, c_rs, 0, 1, mh, nh, accumulate, out_f32, stream);
+}
+
+static int launch_recombine32(int algo, const void* prod, int64_t p_ps, char* C, int64_t c_rs, int64_t c_bs,
+                              int64_t batch, int64_t Mh, int64_t Nh, bool accumulate, hipStream_t stream) {
+    Recombine16Params rp;
+    rp.out_f32 = 1;
+    rp.prod = prod; rp.p_ps = p_ps; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
+    rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
+    dim3 grid((unsigned)ceil_div(Mh * (Nh / 4), 256), (unsigned)batch);
+    if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, stream, rp);
+    else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, stream, rp);
+    return check_launch("recombine32");
+}
+
+// The same five launches for fp32 operands (two Strassen levels, nothing rounded): worth it when
+// the 49 quarter-size products fill the chip with 256 x 256 tiles, because the seven children
+// of the host recursion would each run their own seven products with a partly empty last round.
+static size_t two_level_f32_bytes(int64_t mh, int64_t nh, int64_t kh) {
+    const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
+    return 5 * (align256(mh * kh * 4) + align256(kh * nh * 4)) + 35 * (align256(mq * kq * 4) + align256(kq * nq * 4)) +
+           49 * align256(mq * nq * 4) + 7 * align256(mh * nh * 4);
+}
+
+static bool two_level_f32_shape(int64_t mh, int64_t nh, int64_t kh) {
+    if (mh <= 0 || nh <= 0 || kh <= 0 || mh % 2 || nh % 2 || kh % 2) return false;
+    const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
+    return mq % kBM4 == 0 && nq % kBN4 == 0 && kq % 32 == 0 && 49 * (mq / kBM4) * (nq / kBN4) >= 224;
+}
+
+static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh, int64_t nh, int64_t kh,
+                              bool accumulate, char* ws, hipStream_t stream) {
+    const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
+    const size_t sa1 = align256(mh * kh * 4), sb1 = align256(kh * nh * 4);
+    const size_t sa2 = align256(mq * kq * 4), sb2 = align256(kq * nq * 4);
+    const size_t pb = align256(mq * nq * 4), mb = align256(mh * nh * 4);
+    char* SA1 = ws;
+    char* SB1 = SA1 + 5 * sa1;
+    char* SA2 = SB1 + 5 * sb1;
+    char* SB2 = SA2 + 35 * sa2;
+    char* P = SB2 + 35 * sb2;
+    char* Mp = P + 49 * pb;
+    const bool b_kc = B.rs == 1;
+    {
+        ComboPair pp;
+        const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA, 4);
+        const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB, 4);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos (fp32, level 1)");
+        if (rc) return rc;
+    }
+    View xa1[7], xb1[7];
+    level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1, 4);
+    {
+        ComboMany pm;
+        int64_t most = 0;
+        for (int p = 0; p < 7; ++p) {
+            most = std::max(most, fill_combo(pm.side[2 * p], xa1[p], mq, kq, SA2 + (size_t)p * 5 * sa2, sa2, 5, kStrA, 4));
+            most = std::max(most, fill_combo(pm.side[2 * p + 1], xb1[p], kq, nq, SB2 + (size_t)p * 5 * sb2, sb2, 5, kStrB, 4));
+        }
+        dim3 grid((unsigned)ceil_div(most, 256), 1, 14);
+        hipLaunchKernelGGL(quad_combos_many_f32_kernel, grid, dim3(256), 0, stream, pm);
+        int rc = check_launch("quad_combos (fp32, level 2)");
+        if (rc) return rc;
+    }
+    Gemm2Params g;
+    memset(&g, 0, sizeof(g));
+    for (int p = 0; p < 7; ++p) {
+        View xa2[7], xb2[7];
+        level_operands(STHIP_STRASSEN, xa1[p], xb1[p], mq, nq, kq, SA2 + (size_t)p * 5 * sa2, sa2, SB2 + (size_t)p * 5 * sb2, sb2,
+                       xa2, xb2, 4);
+        for (int j = 0; j < 7; ++j)
+            g.seg[7 * p + j] = Seg2{xa2[j].p, xb2[j].p, xa2[j].rs, b_kc ? xb2[j].cs : xb2[j].rs, 0, 0};
+    }
+    g.C = P; g.c_rs = nq; g.c_ps = (int64_t)(pb / 4); g.c_bs = 0;
+    g.Mh = (int)mq; g.Nh = (int)nq; g.Kh = (int)kq;
+    g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
+    g.out_f32 = 1; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
+    hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, stream);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    int rc = launch_recombine32(STHIP_STRASSEN, P, (int64_t)(pb / 4), Mp, nh, (int64_t)(mb / 4), 7, mq, nq, false, stream);
+    if (rc) return rc;
+    return launch_recombine32(STHIP_STRASSEN, Mp, (int64_t)(mb / 4), C, c_rs, 0, 1, mh, nh, accumulate, stream);
 }
 
 // Vector form of recombine_kernel: four consecutive columns per thread (nh % 4 == 0, C with unit
@@ -1023,6 +1107,7 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
     // two levels may run as one 49-product launch (two_level_flat) or, if the call's layout or
     // result type rules that out, as the host recursion: room for either
     if (levels == 2 && two_level_shape(dt, mh, nh, kh)) return std::max(recursive, two_level_bytes(mh, nh, kh));
+    if (levels == 2 && dt == STHIP_F32 && two_level_f32_shape(mh, nh, kh)) return std::max(recursive, two_level_f32_bytes(mh, nh, kh));
     return recursive;
 }
 
@@ -1049,6 +1134,11 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1) && ws && aligned_to(ws, 256) &&
         ws_bytes >= two_level_bytes(mh, nh, kh))
         return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, stream);
+    if (levels == 2 && (g_stages & 8) && dt == STHIP_F32 && algo == STHIP_STRASSEN && two_level_f32_shape(mh, nh, kh) &&
+        M == Mp && N == Np && K == Kp && c_cs == 1 && c_rs % 4 == 0 && aligned_to(C, 16) && A.cs == 1 &&
+        combos_ok(A, mh, kh, 4) && combos_ok(B, kh, nh, 4) && ws && aligned_to(ws, 256) &&
+        ws_bytes >= two_level_f32_bytes(mh, nh, kh))
+        return two_level_flat_f32(A, B, C, c_rs, mh, nh, kh, accumulate, ws, stream);
     // Whole, aligned problems: all five sums of each operand in one bandwidth-bound launch.
     const bool whole = M == Mp && N == Np && K == Kp;
     const bool vec = whole && combos_ok(A, mh, kh, (int)es) && combos_ok(B, kh, nh, (int)es);
