@@ -49,6 +49,9 @@ WORKLOADS = {
     "strassen1_1024_f32": (1, 1024, 1024, 1024, torch.float32, "strassen", 1),
     "winograd_b8_4096x8192x4096_bf16": (8, 4096, 4096, 8192, torch.bfloat16, "winograd", 1),
     "strassen1_16384_bf16": (1, 16384, 16384, 16384, torch.bfloat16, "strassen", 1),
+    "strassen1_8192_f32": (1, 8192, 8192, 8192, torch.float32, "strassen", 1),
+    "strassen2_16384_f32": (1, 16384, 16384, 16384, torch.float32, "strassen", 2),
+    "classic_8192_f32": (1, 8192, 8192, 8192, torch.float32, "classic", 0),
     "copy_1gib": None,
 }
 DT_NAME = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
