@@ -503,7 +503,7 @@ static size_t f32_batched_bytes(int64_t Mh, int64_t Nh, int64_t Kh) {
 static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
                                  bool accumulate, char* ws, hipStream_t stream);
 static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 bool accumulate, char* ws, hipStream_t stream);
+                                 int algo, bool accumulate, char* ws, hipStream_t stream);
 
 static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                         int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
@@ -577,9 +577,9 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
             return STHIP_OK;
         }
-        if (algo == STHIP_STRASSEN && batch == 1 && 7 * tiles4 >= 224 && ws && aligned_to(ws, 256) &&
+        if (split && batch == 1 && 7 * tiles4 >= 224 && ws && aligned_to(ws, 256) &&
             ws_bytes >= f32_batched_bytes(Mh, Nh, Kh))
-            return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, stream);
+            return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, algo, accumulate, ws, stream);
     }
     // fp32, one Strassen level: run the seven products side by side as a batch (see
     // one_level_f32_batched).  Measured against the fused kernel: 5 x faster at 1024^3 (one product
@@ -1050,35 +1050,32 @@ static const Term kBTerms[7] = {{0, 3, +1}, {0, 0, 0}, {1, 3, -1}, {2, 0, -1}, {
 static const int kSumA[7] = {2, 1, -1, -1, 0, 4, 3};
 static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
 
-// fp32, one Strassen level on the 256 x 256 kernel: the ten quadrant sums in one launch, the
-// seven products (reference numbering M1..M7, raw quadrants read in place) as one grouped launch
-// into seven dense fp32 matrices, one recombination pass.  Nothing is rounded anywhere.
+// fp32, one Strassen or Winograd level on the 256 x 256 kernel: the quadrant sums in one launch,
+// the seven products (raw quadrants read in place) as one grouped launch into seven dense fp32
+// matrices, one recombination pass.  Nothing is rounded anywhere.
 static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 bool accumulate, char* ws, hipStream_t stream) {
+                                 int algo, bool accumulate, char* ws, hipStream_t stream) {
     const size_t sa = align256(Mh * Kh * 4), sb = align256(Kh * Nh * 4), sm = align256(Mh * Nh * 4);
     char* SA = ws;
     char* SB = SA + 5 * sa;
     char* Mbuf = SB + 5 * sb;
-    ComboPair pp;
-    const int64_t na = fill_combo(pp.side[0], A, Mh, Kh, SA, sa, 5, kStrA, 4);
-    const int64_t nb = fill_combo(pp.side[1], B, Kh, Nh, SB, sb, 5, kStrB, 4);
-    dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+    const bool strassen = algo == STHIP_STRASSEN;
+    const int nout = strassen ? 5 : 4;
     if (g_stages & 1) {
+        ComboPair pp;
+        const int64_t na = fill_combo(pp.side[0], A, Mh, Kh, SA, sa, nout, strassen ? kStrA : kWinA, 4);
+        const int64_t nb = fill_combo(pp.side[1], B, Kh, Nh, SB, sb, nout, strassen ? kStrB : kWinB, 4);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
         hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
         int rc = check_launch("quad_combos (fp32)");
         if (rc) return rc;
     }
     const bool b_kc = B.rs == 1;
+    View xa[7], xb[7];
+    level_operands(algo, A, B, Mh, Nh, Kh, SA, sa, SB, sb, xa, xb, 4);
     Gemm2Params g;
     memset(&g, 0, sizeof(g));
-    for (int q = 0; q < 7; ++q) {
-        const Term ta = kATerms[q], tb = kBTerms[q];
-        const char* a = kSumA[q] < 0 ? A.p + ((int64_t)(ta.a >> 1) * Mh * A.rs + (int64_t)(ta.a & 1) * Kh) * 4 : SA + (size_t)kSumA[q] * sa;
-        const int64_t a_ld = kSumA[q] < 0 ? A.rs : Kh;
-        const char* b = kSumB[q] < 0 ? B.p + ((int64_t)(tb.a >> 1) * Kh * B.rs + (int64_t)(tb.a & 1) * Nh * B.cs) * 4 : SB + (size_t)kSumB[q] * sb;
-        const int64_t b_ld = kSumB[q] < 0 ? (b_kc ? B.cs : B.rs) : (b_kc ? Kh : Nh);   // sums keep B's storage orientation
-        g.seg[q] = Seg2{a, b, a_ld, b_ld, 0, 0};
-    }
+    for (int q = 0; q < 7; ++q) g.seg[q] = Seg2{xa[q].p, xb[q].p, xa[q].rs, b_kc ? xb[q].cs : xb[q].rs, 0, 0};
     g.C = Mbuf; g.c_rs = Nh; g.c_ps = (int64_t)(sm / 4); g.c_bs = 0;
     g.Mh = (int)Mh; g.Nh = (int)Nh; g.Kh = (int)Kh;
     g.tiles_m = (int)(Mh / kBM4); g.tiles_n = (int)(Nh / kBN4);
@@ -1088,8 +1085,7 @@ static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t 
         if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
     }
     if (!(g_stages & 4)) return STHIP_OK;
-    return recombine(STHIP_F32, C, c_rs, 1, reinterpret_cast<const float*>(Mbuf), (int64_t)(sm / 4), Mh, Nh, 2 * Mh, 2 * Nh,
-                     accumulate, stream);
+    return launch_recombine32(algo, Mbuf, (int64_t)(sm / 4), C, c_rs, 0, 1, Mh, Nh, accumulate, stream);
 }
 
 static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels) {

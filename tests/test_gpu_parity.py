@@ -403,6 +403,7 @@ def test_large_tile_store_alignment(hip, monkeypatch, dtype, pad, off, algo, lev
     ("classic", 0, (4096, 4096, 96), 1),       # 256 tiles of 256 x 256
     ("classic", 0, (2048, 2048, 64), 4),       # the batch fills the chip
     ("strassen", 1, (4096, 2048, 128), 1),     # seven grouped products of 2048 x 1024 x 64
+    ("winograd", 1, (4096, 2048, 128), 1),
     ("strassen", 2, (8192, 4096, 256), 1),     # the children of the host recursion take the same path
 ])
 def test_fp32_large_tile_exact(hip, algo, levels, shape, batch, tb):
