@@ -15,9 +15,10 @@ namespace sthip {
 
 static thread_local char g_err[512] = "";
 // Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
-// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch.  Only the
-// profiling hook sthip_debug_set_stages changes it.
-static int g_stages = 15;
+// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch, bit 4 = that
+// form recombines 49 -> C in one pass instead of two.  Only the profiling hook
+// sthip_debug_set_stages changes it.
+static int g_stages = 31;
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -277,6 +278,106 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
         }
         __builtin_nontemporal_store(w, d);
     }
+}
+
+// Both recombinations of a two-level product in one pass: from the 49 quarter-size 16-bit products
+// (first-level product p, second-level product k at prod + (7 p + k) * p_ps) straight to C.  The
+// second-level result of every first-level product is rounded to the operand type in registers,
+// exactly where the two-pass form stores it, and the first level adds in the same order as
+// recombine16_kernel (p visited in the order 4 6 5 2 0 3 1 gives each quadrant its terms in that
+// order), so the result is bit-identical to the two passes -- without writing and re-reading the
+// seven half-size products.  One thread per 16-byte chunk of a quarter-size row; Mh, Nh are the
+// quarter sizes here.
+template <class T>
+__device__ __forceinline__ float round16(float x) {
+    if constexpr (__is_same(T, bf16_t)) return bf16lo(pack_bf16(x, 0.f));
+    else return (float)as_f16x2(pack_f16(x, 0.f))[0];
+}
+
+template <class T, int ALGO2>
+__global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Params p) {
+    const int nq = p.Nh / 8;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.Mh * nq) return;
+    const int i = (int)(idx / nq), j = (int)(idx % nq) * 8;
+    const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)i * p.Nh + j) * 2;
+    float acc[4][4][8];   // [quadrant of C][quarter block within it][element]
+    // second level of first-level product pp -> m[quarter block][element], rounded to T
+    auto second = [&](int pp, float (&m)[4][8]) {
+        float x[7][8];
+#pragma unroll
+        for (int k = 0; k < 7; ++k)
+            unpack8<T>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (int64_t)(7 * pp + k) * p.p_ps * 2)), x[k]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if constexpr (ALGO2 == STHIP_STRASSEN) {
+                m[0][e] = ((x[4][e] + x[6][e]) - x[2][e]) + x[3][e];
+                m[1][e] = x[0][e] + x[2][e];
+                m[2][e] = x[5][e] + x[6][e];
+                m[3][e] = ((x[4][e] - x[5][e]) + x[0][e]) + x[1][e];
+            } else {
+                const float u2 = x[0][e] + x[2][e], u3 = u2 + x[3][e], u4 = u2 + x[4][e];
+                m[0][e] = x[0][e] + x[1][e];
+                m[1][e] = u4 + x[5][e];
+                m[2][e] = u3 + x[6][e];
+                m[3][e] = u3 + x[4][e];
+            }
+#pragma unroll
+            for (int b = 0; b < 4; ++b) m[b][e] = round16<T>(m[b][e]);
+        }
+    };
+    float m[4][8];
+#define STHIP_EACH for (int b = 0; b < 4; ++b) for (int e = 0; e < 8; ++e)
+    second(4, m);   // M1: C11 = M1 ..., C22 = M1 ...
+#pragma unroll
+    STHIP_EACH { acc[0][b][e] = m[b][e]; acc[3][b][e] = m[b][e]; }
+    second(6, m);   // M4: C11 += M4, C21 = M4
+#pragma unroll
+    STHIP_EACH { acc[0][b][e] += m[b][e]; acc[2][b][e] = m[b][e]; }
+    second(5, m);   // M2: C22 -= M2, C21 += M2
+#pragma unroll
+    STHIP_EACH { acc[3][b][e] -= m[b][e]; acc[2][b][e] += m[b][e]; }
+    second(2, m);   // M5: C11 -= M5, C12 = M5
+#pragma unroll
+    STHIP_EACH { acc[0][b][e] -= m[b][e]; acc[1][b][e] = m[b][e]; }
+    second(0, m);   // M3: C22 += M3, C12 += M3
+#pragma unroll
+    STHIP_EACH { acc[3][b][e] += m[b][e]; acc[1][b][e] += m[b][e]; }
+    second(3, m);   // M7: C11 += M7
+#pragma unroll
+    STHIP_EACH { acc[0][b][e] += m[b][e]; }
+    second(1, m);   // M6: C22 += M6
+#pragma unroll
+    STHIP_EACH { acc[3][b][e] += m[b][e]; }
+#undef STHIP_EACH
+    const int mh = 2 * p.Mh, nh = 2 * p.Nh;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t row = (int64_t)(q >> 1) * mh + (b >> 1) * p.Mh + i, col = (int64_t)(q & 1) * nh + (b & 1) * p.Nh + j;
+            if (p.out_f32) {
+                f32x4* d = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + row * p.c_rs + col);
+                f32x4 lo = {acc[q][b][0], acc[q][b][1], acc[q][b][2], acc[q][b][3]}, hi = {acc[q][b][4], acc[q][b][5], acc[q][b][6], acc[q][b][7]};
+                if (p.accumulate) { lo += d[0]; hi += d[1]; }
+                d[0] = lo; d[1] = hi;
+            } else {
+                u32x4* d = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.C) + (row * p.c_rs + col) * 2);
+                if (p.accumulate) {
+                    float old[8];
+                    unpack8<T>(*d, old);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[q][b][e] += old[e];
+                }
+                u32x4 w;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if constexpr (__is_same(T, bf16_t)) w[k] = pack_bf16(acc[q][b][2 * k], acc[q][b][2 * k + 1]);
+                    else w[k] = pack_f16(acc[q][b][2 * k], acc[q][b][2 * k + 1]);
+                }
+                __builtin_nontemporal_store(w, d);
+            }
+        }
 }
 
 // The same recombination for seven fp32 products (16-bit operands, fp32 result: the products are
@@ -856,10 +957,22 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     }
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
 
-    // 49 -> 7 (second-level recombination, one batch entry per first-level product), then 7 -> C
-    int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
-    if (rc) return rc;
-    return launch_recombine16(dt, STHIP_STRASSEN, Mp, (int64_t)(mb / 2), C, c_rs, 0, 1, mh, nh, accumulate, out_f32, stream);
+    // 49 -> C: both recombinations in one pass (bit 4 of the stage mask off: as two passes, 49 -> 7
+    // with one batch entry per first-level product, then 7 -> C)
+    if (!(g_stages & 16)) {
+        int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
+        if (rc) return rc;
+        return launch_recombine16(dt, STHIP_STRASSEN, Mp, (int64_t)(mb / 2), C, c_rs, 0, 1, mh, nh, accumulate, out_f32, stream);
+    }
+    Recombine16Params rp;
+    rp.prod = P; rp.p_ps = (int64_t)(pb / 2); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
+    rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = out_f32 ? 1 : 0;
+    dim3 grid((unsigned)ceil_div(mq * (nq / 8), 256), 1);
+#define GO(T, A) hipLaunchKernelGGL((recombine16x2_kernel<T, A>), grid, dim3(256), 0, stream, rp)
+    if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
+    else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
+#undef GO
+    return check_launch("recombine16x2");
 }
 
 static int launch_recombine32(int algo, const void* prod, int64_t p_ps, char* C, int64_t c_rs, int64_t c_bs,
@@ -1311,7 +1424,7 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
 
 int sthip_debug_set_stages(int mask) {
     const int old = g_stages;
-    g_stages = mask & 15;
+    g_stages = mask & 31;
     return old;
 }
 

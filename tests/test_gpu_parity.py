@@ -255,6 +255,12 @@ def test_two_levels_as_one_launch(hip, dtype, algo, ta, tb, shape):
         rec = hip.gemm(Ag, Bg, algo=algo, levels=2)
     finally:
         lib.sthip_debug_set_stages(prev)
+    prev = lib.sthip_debug_set_stages(15)   # bit 4 off: 49 -> 7 -> C as two recombination passes
+    try:
+        two_pass = hip.gemm(Ag, Bg, algo=algo, levels=2)
+    finally:
+        lib.sthip_debug_set_stages(prev)
+    assert torch.equal(flat, two_pass)      # the one-pass recombination rounds and adds in the same places
     ref = Ag.double() @ Bg.double()
     rel = lambda X: float(torch.linalg.norm(X.double() - ref) / torch.linalg.norm(ref))
     assert rel(flat) <= TOL[dtype] and rel(rec) <= TOL[dtype]
