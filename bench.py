@@ -189,13 +189,14 @@ def main():
     # the dominant kernel alone: with the pre-pass switched off the grouped GEMM re-uses the
     # quadrant sums the calls above left in the workspace
     kernel_s, prepass_s, recombine_s = ev / args.steps, 0.0, 0.0
-    staged = levels == 1 and algo != "classic" and nbytes > 0
+    staged = levels in (1, 2) and algo != "classic" and nbytes > 0 and (levels == 1 or dtype != torch.float32)
     if staged:
-        all_stages = lib.sthip_debug_set_stages(2)
+        all_stages = lib.sthip_debug_set_stages(0)
+        lib.sthip_debug_set_stages((all_stages & ~7) | 2)   # one stage at a time, the other switches as they were
         _, ev_k = time_gpu(fn, args.steps, 3)
-        lib.sthip_debug_set_stages(1)
+        lib.sthip_debug_set_stages((all_stages & ~7) | 1)
         _, ev_p = time_gpu(fn, args.steps, 3)
-        lib.sthip_debug_set_stages(4)
+        lib.sthip_debug_set_stages((all_stages & ~7) | 4)
         _, ev_r = time_gpu(fn, args.steps, 3)
         lib.sthip_debug_set_stages(all_stages)
         kernel_s, prepass_s, recombine_s = ev_k / args.steps, ev_p / args.steps, ev_r / args.steps

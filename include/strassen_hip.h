@@ -128,8 +128,8 @@ int sthip_debug_transpose_read(void* out, void* stream);
 /* Profiling aid: selects which stages of the pipelined one-level path later calls run
  * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM, bit 2 = recombination pass of the
  * grouped paths; bit 3 lets two-level calls run as one 49-product launch instead of the host
- * recursion, bit 4 lets that form recombine 49 -> C in one pass instead of two; default 31) and
- * returns the previous mask.  With mask 2 the GEMM re-uses the
+ * recursion, bit 4 lets that form recombine 49 -> C in one pass instead of two, bit 5 lets it
+ * form the sums of both levels in one pass instead of two; default 63) and returns the previous mask.  With mask 2 the GEMM re-uses the
  * sums a previous call left in the same workspace, so the dominant kernel can be timed alone.
  * Process-wide; not for production calls.  No counterpart in the reference. */
 int sthip_debug_set_stages(int mask);

@@ -16,9 +16,9 @@ namespace sthip {
 static thread_local char g_err[512] = "";
 // Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
 // bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch, bit 4 = that
-// form recombines 49 -> C in one pass instead of two.  Only the profiling hook
-// sthip_debug_set_stages changes it.
-static int g_stages = 31;
+// form recombines 49 -> C in one pass instead of two, bit 5 = and forms the sums of both levels in
+// one pass instead of two.  Only the profiling hook sthip_debug_set_stages changes it.
+static int g_stages = 63;
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -179,6 +179,119 @@ template <class T>
 __global__ void __launch_bounds__(256) quad_combos_many_kernel(const ComboMany pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
 __global__ void __launch_bounds__(256) quad_combos_many_f32_kernel(const ComboMany pp) { quad_combos_f32_body(pp.side[blockIdx.z]); }
 
+// Eight 16-bit elements of a 16-byte chunk as floats.
+template <class T>
+__device__ __forceinline__ void unpack8(const u32x4 v, float* x) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if constexpr (__is_same(T, bf16_t)) { x[2 * w] = bf16lo(v[w]); x[2 * w + 1] = bf16hi(v[w]); }
+        else { const f16x2 h = as_f16x2(v[w]); x[2 * w] = (float)h[0]; x[2 * w + 1] = (float)h[1]; }
+    }
+}
+
+// NW 32-bit words (2 NW 16-bit elements) as floats, and back with one rounding.
+template <int NW> struct WordVec;
+template <> struct WordVec<2> { typedef u32x2 type; };
+template <> struct WordVec<4> { typedef u32x4 type; };
+template <class T, int NW>
+__device__ __forceinline__ void unpack_words(const typename WordVec<NW>::type v, float* x) {
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        if constexpr (__is_same(T, bf16_t)) { x[2 * w] = bf16lo(v[w]); x[2 * w + 1] = bf16hi(v[w]); }
+        else { const f16x2 h = as_f16x2(v[w]); x[2 * w] = (float)h[0]; x[2 * w + 1] = (float)h[1]; }
+    }
+}
+template <class T, int NW>
+__device__ __forceinline__ typename WordVec<NW>::type pack_words(const float* x) {
+    typename WordVec<NW>::type w;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        if constexpr (__is_same(T, bf16_t)) w[i] = pack_bf16(x[2 * i], x[2 * i + 1]);
+        else w[i] = pack_f16(x[2 * i], x[2 * i + 1]);
+    }
+    return w;
+}
+// Elements per thread of the two-level passes: four (8-byte accesses) keep their register use low
+// enough for four or more waves per SIMD; with eight the kernels ran at one or two.
+constexpr int kNW2 = 2, kEPT2 = 2 * kNW2;
+
+// The sums of BOTH levels of a two-level product for one operand in one pass: the sixteen quarter
+// blocks are read once; every first-level operand (a quadrant, or a sum of two rounded to the
+// operand type as the two-pass form stores it) is formed in registers, the quarters of the
+// first-level sums that the second level multiplies directly are stored, and so are the
+// second-level sums of all seven first-level operands.  Same additions in the same order as
+// quad_combos_body, so the outputs are bit-identical to the two passes -- without writing the
+// other half of the first-level sums and without re-reading any of them.
+struct Combo2Params {
+    const void* x[16];        // quarter blocks of the operand, logical (R, C) -> x[4 R + C]
+    void* s1[5];              // first-level sums: dense half-size blocks in the operand's storage orientation
+    void* s2[7];              // second-level sums of first-level operand p: s2[p] + o * s2_stride bytes
+    int64_t s2_stride;
+    int64_t ld_in, ld1, ld2;  // elements
+    int64_t q1_u, q1_v;       // element offset of quarter (u, v) inside a first-level sum: u * q1_u + v * q1_v
+    int rows, chunks_per_row; // of one quarter block, storage order
+    int nout2, keep;          // second-level sums per operand; quarters (bit 2 u + v) of the first-level sums to store
+    signed char l1[7][4];     // first-level operand p over the quadrants 11 12 21 22 (a unit vector = that quadrant)
+    signed char l1_sum[7];    // index into s1 if p is a sum, -1 if it is a quadrant
+    signed char c2[5][4];     // second-level sums over the four quarters of a first-level operand
+};
+struct Combo2Pair { Combo2Params side[2]; };
+
+template <class T>
+__global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) {
+    typedef typename WordVec<kNW2>::type vec_t;
+    const Combo2Params& p = pp.side[blockIdx.z];
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
+    const int r = (int)(idx / p.chunks_per_row), c = (int)(idx % p.chunks_per_row);
+    const int64_t in_off = ((int64_t)r * p.ld_in + c * kEPT2) * 2;
+    const int64_t o1 = (int64_t)r * p.ld1 + c * kEPT2, o2 = ((int64_t)r * p.ld2 + c * kEPT2) * 2;
+    vec_t v[16];
+#pragma unroll
+    for (int b = 0; b < 16; ++b)
+        v[b] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(reinterpret_cast<const char*>(p.x[b]) + in_off));
+    for (int q = 0; q < 7; ++q) {
+        // quarters (u, v) of first-level operand q
+        vec_t s[4];
+#pragma unroll
+        for (int uv = 0; uv < 4; ++uv) {
+            float acc[kEPT2];
+#pragma unroll
+            for (int e = 0; e < kEPT2; ++e) acc[e] = 0.f;
+#pragma unroll
+            for (int Q = 0; Q < 4; ++Q) {
+                const int cf = p.l1[q][Q];
+                if (cf == 0) continue;
+                float x[kEPT2];
+                unpack_words<T, kNW2>(v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)], x);
+#pragma unroll
+                for (int e = 0; e < kEPT2; ++e) acc[e] = cf > 0 ? acc[e] + x[e] : acc[e] - x[e];
+            }
+            s[uv] = pack_words<T, kNW2>(acc);   // exact for a single quadrant, the one rounding of a sum otherwise
+            const int dst = p.l1_sum[q];
+            if (dst >= 0 && ((p.keep >> uv) & 1))
+                __builtin_nontemporal_store(s[uv], reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s1[dst]) + ((uv >> 1) * p.q1_u + (uv & 1) * p.q1_v + o1) * 2));
+        }
+        float x[4][kEPT2];
+#pragma unroll
+        for (int uv = 0; uv < 4; ++uv) unpack_words<T, kNW2>(s[uv], x[uv]);
+        for (int o = 0; o < p.nout2; ++o) {
+            float acc[kEPT2];
+#pragma unroll
+            for (int e = 0; e < kEPT2; ++e) {
+                float a = 0.f;
+#pragma unroll
+                for (int uv = 0; uv < 4; ++uv) {
+                    const int cf = p.c2[o][uv];
+                    if (cf > 0) a += x[uv][e]; else if (cf < 0) a -= x[uv][e];
+                }
+                acc[e] = a;
+            }
+            __builtin_nontemporal_store(pack_words<T, kNW2>(acc), reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s2[q]) + (int64_t)o * p.s2_stride + o2));
+        }
+    }
+}
+
 // Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
 // Strassen (fixed_strassen.py:88-97): A side S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.
 static const signed char kStrA[5][4] = {{1, 1, 0, 0}, {0, 0, 1, 1}, {1, 0, 0, 1}, {0, 1, 0, -1}, {-1, 0, 1, 0}};
@@ -213,14 +326,6 @@ struct Recombine16Params {
     int out_f32;          // C is fp32 (no final rounding) instead of the operand type
 };
 
-template <class T>
-__device__ __forceinline__ void unpack8(const u32x4 v, float* x) {
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        if constexpr (__is_same(T, bf16_t)) { x[2 * w] = bf16lo(v[w]); x[2 * w + 1] = bf16hi(v[w]); }
-        else { const f16x2 h = as_f16x2(v[w]); x[2 * w] = (float)h[0]; x[2 * w + 1] = (float)h[1]; }
-    }
-}
 
 template <class T, int ALGO>
 __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Params p) {
@@ -296,20 +401,22 @@ __device__ __forceinline__ float round16(float x) {
 
 template <class T, int ALGO2>
 __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Params p) {
-    const int nq = p.Nh / 8;
+    typedef typename WordVec<kNW2>::type vec_t;
+    constexpr int E = kEPT2;
+    const int nq = p.Nh / E;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.Mh * nq) return;
-    const int i = (int)(idx / nq), j = (int)(idx % nq) * 8;
+    const int i = (int)(idx / nq), j = (int)(idx % nq) * E;
     const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)i * p.Nh + j) * 2;
-    float acc[4][4][8];   // [quadrant of C][quarter block within it][element]
+    float acc[4][4][E];   // [quadrant of C][quarter block within it][element]
     // second level of first-level product pp -> m[quarter block][element], rounded to T
-    auto second = [&](int pp, float (&m)[4][8]) {
-        float x[7][8];
+    auto second = [&](int pp, float (&m)[4][E]) {
+        float x[7][E];
 #pragma unroll
         for (int k = 0; k < 7; ++k)
-            unpack8<T>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (int64_t)(7 * pp + k) * p.p_ps * 2)), x[k]);
+            unpack_words<T, kNW2>(__builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + (int64_t)(7 * pp + k) * p.p_ps * 2)), x[k]);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < E; ++e) {
             if constexpr (ALGO2 == STHIP_STRASSEN) {
                 m[0][e] = ((x[4][e] + x[6][e]) - x[2][e]) + x[3][e];
                 m[1][e] = x[0][e] + x[2][e];
@@ -326,8 +433,8 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
             for (int b = 0; b < 4; ++b) m[b][e] = round16<T>(m[b][e]);
         }
     };
-    float m[4][8];
-#define STHIP_EACH for (int b = 0; b < 4; ++b) for (int e = 0; e < 8; ++e)
+    float m[4][E];
+#define STHIP_EACH for (int b = 0; b < 4; ++b) for (int e = 0; e < E; ++e)
     second(4, m);   // M1: C11 = M1 ..., C22 = M1 ...
 #pragma unroll
     STHIP_EACH { acc[0][b][e] = m[b][e]; acc[3][b][e] = m[b][e]; }
@@ -357,25 +464,23 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
         for (int b = 0; b < 4; ++b) {
             const int64_t row = (int64_t)(q >> 1) * mh + (b >> 1) * p.Mh + i, col = (int64_t)(q & 1) * nh + (b & 1) * p.Nh + j;
             if (p.out_f32) {
-                f32x4* d = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.C) + row * p.c_rs + col);
-                f32x4 lo = {acc[q][b][0], acc[q][b][1], acc[q][b][2], acc[q][b][3]}, hi = {acc[q][b][4], acc[q][b][5], acc[q][b][6], acc[q][b][7]};
-                if (p.accumulate) { lo += d[0]; hi += d[1]; }
-                d[0] = lo; d[1] = hi;
+                float* d = reinterpret_cast<float*>(p.C) + row * p.c_rs + col;
+#pragma unroll
+                for (int e = 0; e < E; e += 4) {
+                    f32x4 o = {acc[q][b][e], acc[q][b][e + 1], acc[q][b][e + 2], acc[q][b][e + 3]};
+                    f32x4* dd = reinterpret_cast<f32x4*>(d + e);
+                    if (p.accumulate) o += *dd;
+                    *dd = o;
+                }
             } else {
-                u32x4* d = reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.C) + (row * p.c_rs + col) * 2);
+                vec_t* d = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.C) + (row * p.c_rs + col) * 2);
                 if (p.accumulate) {
-                    float old[8];
-                    unpack8<T>(*d, old);
+                    float old[E];
+                    unpack_words<T, kNW2>(*d, old);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[q][b][e] += old[e];
+                    for (int e = 0; e < E; ++e) acc[q][b][e] += old[e];
                 }
-                u32x4 w;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    if constexpr (__is_same(T, bf16_t)) w[k] = pack_bf16(acc[q][b][2 * k], acc[q][b][2 * k + 1]);
-                    else w[k] = pack_f16(acc[q][b][2 * k], acc[q][b][2 * k + 1]);
-                }
-                __builtin_nontemporal_store(w, d);
+                __builtin_nontemporal_store(pack_words<T, kNW2>(acc[q][b]), d);
             }
         }
 }
@@ -873,6 +978,47 @@ static int launch_recombine16(int dt, int algo, const void* prod, int64_t p_ps, 
 // those into C.  Every level returns its result in the operand type, as the reference's
 // recursion does (fixed_strassen_fp32_agg.py:47-50); the first level is always Strassen.
 // Needs: 16-bit operands, whole aligned problem, C in the operand type with 16-byte aligned rows.
+// One operand of quad_combos2_kernel.  X is the whole operand, (rq, cq) the quarter-block size in
+// its logical (row, col) indexing; side 0 = A, 1 = B; first level Strassen, second level `algo2`.
+// S1 / S2 are laid out as the two-pass form lays them out (S1: five dense half-size sums s1_b
+// bytes apart; S2: for first-level operand p the sums at S2 + (5 p + o) * s2_b).
+static int64_t fill_combo2(Combo2Params& cp, View X, int64_t rq, int64_t cq, char* S1, size_t s1_b, char* S2, size_t s2_b,
+                           int side, int algo2) {
+    memset(&cp, 0, sizeof(cp));
+    const bool row_major = X.cs == 1;
+    for (int R = 0; R < 4; ++R)
+        for (int C = 0; C < 4; ++C) cp.x[4 * R + C] = X.p + ((int64_t)R * rq * X.rs + (int64_t)C * cq * X.cs) * 2;
+    // first-level operands in kernel order (level_operands): A side A11 S9 S2 S7 S5 S3 A22 with the
+    // sums numbered as the outputs of kStrA (S2 S3 S5 S7 S9 = 0..4); B side S1 S10 B22 S8 S6 B11 S4
+    // (kStrB: S1 S4 S6 S8 S10 = 0..4)
+    static const signed char kFirstA[7] = {-1, 4, 0, 3, 2, 1, -4}, kFirstB[7] = {0, 4, -4, 3, 2, -1, 1};   // >= 0: sum; -1 - q: quadrant q
+    for (int p = 0; p < 7; ++p) {
+        const int f = side == 0 ? kFirstA[p] : kFirstB[p];
+        cp.l1_sum[p] = (signed char)(f >= 0 ? f : -1);
+        for (int Q = 0; Q < 4; ++Q)
+            cp.l1[p][Q] = f >= 0 ? (side == 0 ? kStrA[f][Q] : kStrB[f][Q]) : (Q == -1 - f ? 1 : 0);
+        cp.s2[p] = S2 + (size_t)p * 5 * s2_b;
+    }
+    for (int o = 0; o < 5; ++o) cp.s1[o] = S1 + (size_t)o * s1_b;
+    cp.s2_stride = (int64_t)s2_b;
+    const bool strassen2 = algo2 == STHIP_STRASSEN;
+    cp.nout2 = strassen2 ? 5 : 4;
+    for (int o = 0; o < cp.nout2; ++o)
+        for (int uv = 0; uv < 4; ++uv)
+            cp.c2[o][uv] = strassen2 ? (side == 0 ? kStrA[o][uv] : kStrB[o][uv]) : (side == 0 ? kWinA[o][uv] : kWinB[o][uv]);
+    // quarters of a first-level sum that the second level multiplies as they are (level_operands):
+    // Strassen 11 and 22; Winograd 11, 12 and 22 of an A-side operand, 11, 21 and 22 of a B-side one
+    cp.keep = strassen2 ? 0x9 : (side == 0 ? 0xB : 0xD);
+    const int64_t rows = row_major ? rq : cq, cols = row_major ? cq : rq;   // quarter block, storage order
+    cp.ld_in = row_major ? X.rs : X.cs;
+    cp.ld1 = 2 * cols;
+    cp.ld2 = cols;
+    cp.q1_u = row_major ? rq * cp.ld1 : rq;
+    cp.q1_v = row_major ? cq : cq * cp.ld1;
+    cp.rows = (int)rows; cp.chunks_per_row = (int)(cols / kEPT2);
+    return rows * (cols / kEPT2);
+}
+
 static size_t two_level_bytes(int64_t mh, int64_t nh, int64_t kh) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     return 5 * (align256(mh * kh * 2) + align256(kh * nh * 2)) + 35 * (align256(mq * kq * 2) + align256(kq * nq * 2)) +
@@ -898,8 +1044,19 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     const bool a_kc = A.cs == 1, b_kc = B.rs == 1;
     const int nout2 = algo == STHIP_STRASSEN ? 5 : 4;
 
+    // sums of both levels in one pass (bit 5 of the stage mask off: as two passes)
+    if ((g_stages & 32) && (g_stages & 1)) {
+        Combo2Pair pp;
+        const int64_t na = fill_combo2(pp.side[0], A, mq, kq, SA1, sa1, SA2, sa2, 0, algo);
+        const int64_t nb = fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, algo);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
+        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos2");
+        if (rc) return rc;
+    }
     // first-level sums (Strassen)
-    {
+    if (!(g_stages & 32) && (g_stages & 1)) {
         ComboPair pp;
         const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA);
         const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB);
@@ -913,7 +1070,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1);
 
     // second-level sums of all fourteen operands
-    {
+    if (!(g_stages & 32) && (g_stages & 1)) {
         ComboMany pm;
         int64_t most = 0;
         for (int p = 0; p < 7; ++p) {
@@ -943,8 +1100,9 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     g.out_f32 = 0; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
     const LaunchTable3* t4 = table4_for(dt);
     const bool big = a_kc && t4 && mq % kBM4 == 0 && nq % kBN4 == 0 && kq >= 1024 && forced_tile() != 5 && forced_tile() != 2;
-    hipError_t e;
-    if (big) {
+    hipError_t e = hipSuccess;
+    if (!(g_stages & 2)) {
+    } else if (big) {
         g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
         g.c_wide = wide_rows(g.C, g.c_rs, g.c_ps, 0);
         e = t4->fn[b_kc ? 1 : 0](g, 1, stream);
@@ -959,6 +1117,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
 
     // 49 -> C: both recombinations in one pass (bit 4 of the stage mask off: as two passes, 49 -> 7
     // with one batch entry per first-level product, then 7 -> C)
+    if (!(g_stages & 4)) return STHIP_OK;
     if (!(g_stages & 16)) {
         int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
         if (rc) return rc;
@@ -967,7 +1126,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     Recombine16Params rp;
     rp.prod = P; rp.p_ps = (int64_t)(pb / 2); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
     rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = out_f32 ? 1 : 0;
-    dim3 grid((unsigned)ceil_div(mq * (nq / 8), 256), 1);
+    dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
 #define GO(T, A) hipLaunchKernelGGL((recombine16x2_kernel<T, A>), grid, dim3(256), 0, stream, rp)
     if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
     else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
@@ -1424,7 +1583,7 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
 
 int sthip_debug_set_stages(int mask) {
     const int old = g_stages;
-    g_stages = mask & 31;
+    g_stages = mask & 63;
     return old;
 }
 
