@@ -63,10 +63,10 @@ enum sthip_algo {
  * 256 x 256 tiles when A is contiguous along k and the blocks are multiples of 256 and large
  * enough to fill the chip, else batched over dense operand copies); nothing is rounded.  Plain
  * products (STHIP_CLASSIC) of all three types take the 256 x 256 kernel under the same conditions.
- * levels = 2 on tile-aligned 16-bit problems runs as five launches (sums of both levels, ONE
- * grouped GEMM of the 49 quarter-size products, two recombination passes; every level returns
+ * levels = 2 on tile-aligned 16-bit problems runs as three launches (the sums of both levels,
+ * ONE grouped GEMM of the 49 quarter-size products, both recombinations; every level returns
  * its products in the operand type, the first level is always Strassen); large fp32 Strassen
- * problems have the same form with nothing rounded.  Otherwise levels >= 2 recurses on the host
+ * problems run as five (sums, sums, the 49 products, two recombinations) with nothing rounded.  Otherwise levels >= 2 recurses on the host
  * (sums and products of the upper levels in workspace) and requires the workspace.
  *
  * Replaces: _strassen_base (fixed_strassen.py:11-57, fixed_strassen_fp32_agg.py:12-56),

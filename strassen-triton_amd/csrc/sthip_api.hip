@@ -971,13 +971,6 @@ static int launch_recombine16(int dt, int algo, const void* prod, int64_t p_ps, 
     return check_launch("recombine16");
 }
 
-// Two levels as five launches: sums of the first level, sums of the second level for all seven
-// first-level products at once, ONE grouped GEMM of the 49 quarter-size products (the schedule
-// the reference's two-layer Triton kernel runs per tile, strassen.py:373-611, here on whole
-// matrices), recombination of the 49 into the seven first-level products, recombination of
-// those into C.  Every level returns its result in the operand type, as the reference's
-// recursion does (fixed_strassen_fp32_agg.py:47-50); the first level is always Strassen.
-// Needs: 16-bit operands, whole aligned problem, C in the operand type with 16-byte aligned rows.
 // One operand of quad_combos2_kernel.  X is the whole operand, (rq, cq) the quarter-block size in
 // its logical (row, col) indexing; side 0 = A, 1 = B; first level Strassen, second level `algo2`.
 // S1 / S2 are laid out as the two-pass form lays them out (S1: five dense half-size sums s1_b
@@ -1019,6 +1012,14 @@ static int64_t fill_combo2(Combo2Params& cp, View X, int64_t rq, int64_t cq, cha
     return rows * (cols / kEPT2);
 }
 
+// Two levels as three launches: the sums of both levels in one pass over the operands, ONE
+// grouped GEMM of the 49 quarter-size products (the schedule the reference's two-layer Triton
+// kernel runs per tile, strassen.py:373-611, here on whole matrices), both recombinations in one
+// pass.  Every level returns its result in the operand type, as the reference's recursion does
+// (fixed_strassen_fp32_agg.py:47-50): the passes round in registers where the five-launch form
+// (sums 1, sums 2, GEMM, 49 -> 7, 7 -> C; stage-mask bits 4 and 5 off) rounds on its way through
+// memory, and give the same bits.  The first level is always Strassen.
+// Needs: 16-bit operands, whole aligned problem, C in the operand type with 16-byte aligned rows.
 static size_t two_level_bytes(int64_t mh, int64_t nh, int64_t kh) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     return 5 * (align256(mh * kh * 2) + align256(kh * nh * 2)) + 35 * (align256(mq * kq * 2) + align256(kq * nq * 2)) +
@@ -1146,7 +1147,8 @@ static int launch_recombine32(int algo, const void* prod, int64_t p_ps, char* C,
     return check_launch("recombine32");
 }
 
-// The same five launches for fp32 operands (two Strassen levels, nothing rounded): worth it when
+// Two levels of fp32 operands as five launches (sums 1, sums 2, one grouped GEMM of the 49
+// products, 49 -> 7, 7 -> C; two Strassen levels, nothing rounded): worth it when
 // the 49 quarter-size products fill the chip with 256 x 256 tiles, because the seven children
 // of the host recursion would each run their own seven products with a partly empty last round.
 static size_t two_level_f32_bytes(int64_t mh, int64_t nh, int64_t kh) {
