@@ -193,6 +193,9 @@ __device__ __forceinline__ void unpack8(const u32x4 v, float* x) {
 template <int NW> struct WordVec;
 template <> struct WordVec<2> { typedef u32x2 type; };
 template <> struct WordVec<4> { typedef u32x4 type; };
+// kEPT2 elements of type T as one vector load / store: 8 bytes of 16-bit elements, 16 bytes of fp32
+template <class T> struct ElemVec { typedef u32x2 type; };
+template <> struct ElemVec<float> { typedef f32x4 type; };
 template <class T, int NW>
 __device__ __forceinline__ void unpack_words(const typename WordVec<NW>::type v, float* x) {
 #pragma unroll
@@ -214,6 +217,16 @@ __device__ __forceinline__ typename WordVec<NW>::type pack_words(const float* x)
 // Elements per thread of the two-level passes: four (8-byte accesses) keep their register use low
 // enough for four or more waves per SIMD; with eight the kernels ran at one or two.
 constexpr int kNW2 = 2, kEPT2 = 2 * kNW2;
+template <class T>
+__device__ __forceinline__ void unpack_elems(const typename ElemVec<T>::type v, float* x) {
+    if constexpr (__is_same(T, float)) { x[0] = v[0]; x[1] = v[1]; x[2] = v[2]; x[3] = v[3]; }
+    else unpack_words<T, kNW2>(v, x);
+}
+template <class T>
+__device__ __forceinline__ typename ElemVec<T>::type pack_elems(const float* x) {
+    if constexpr (__is_same(T, float)) { f32x4 v = {x[0], x[1], x[2], x[3]}; return v; }
+    else return pack_words<T, kNW2>(x);
+}
 
 // The sums of BOTH levels of a two-level product for one operand in one pass: the sixteen quarter
 // blocks are read once; every first-level operand (a quadrant, or a sum of two rounded to the
@@ -239,13 +252,14 @@ struct Combo2Pair { Combo2Params side[2]; };
 
 template <class T>
 __global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) {
-    typedef typename WordVec<kNW2>::type vec_t;
+    typedef typename ElemVec<T>::type vec_t;
+    constexpr int ES = (int)sizeof(T) == 4 ? 4 : 2;
     const Combo2Params& p = pp.side[blockIdx.z];
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
     const int r = (int)(idx / p.chunks_per_row), c = (int)(idx % p.chunks_per_row);
-    const int64_t in_off = ((int64_t)r * p.ld_in + c * kEPT2) * 2;
-    const int64_t o1 = (int64_t)r * p.ld1 + c * kEPT2, o2 = ((int64_t)r * p.ld2 + c * kEPT2) * 2;
+    const int64_t in_off = ((int64_t)r * p.ld_in + c * kEPT2) * ES;
+    const int64_t o1 = (int64_t)r * p.ld1 + c * kEPT2, o2 = ((int64_t)r * p.ld2 + c * kEPT2) * ES;
     vec_t v[16];
 #pragma unroll
     for (int b = 0; b < 16; ++b)
@@ -263,18 +277,18 @@ __global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) 
                 const int cf = p.l1[q][Q];
                 if (cf == 0) continue;
                 float x[kEPT2];
-                unpack_words<T, kNW2>(v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)], x);
+                unpack_elems<T>(v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)], x);
 #pragma unroll
                 for (int e = 0; e < kEPT2; ++e) acc[e] = cf > 0 ? acc[e] + x[e] : acc[e] - x[e];
             }
-            s[uv] = pack_words<T, kNW2>(acc);   // exact for a single quadrant, the one rounding of a sum otherwise
+            s[uv] = pack_elems<T>(acc);   // exact for a single quadrant, the one rounding of a sum otherwise
             const int dst = p.l1_sum[q];
             if (dst >= 0 && ((p.keep >> uv) & 1))
-                __builtin_nontemporal_store(s[uv], reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s1[dst]) + ((uv >> 1) * p.q1_u + (uv & 1) * p.q1_v + o1) * 2));
+                __builtin_nontemporal_store(s[uv], reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s1[dst]) + ((uv >> 1) * p.q1_u + (uv & 1) * p.q1_v + o1) * ES));
         }
         float x[4][kEPT2];
 #pragma unroll
-        for (int uv = 0; uv < 4; ++uv) unpack_words<T, kNW2>(s[uv], x[uv]);
+        for (int uv = 0; uv < 4; ++uv) unpack_elems<T>(s[uv], x[uv]);
         for (int o = 0; o < p.nout2; ++o) {
             float acc[kEPT2];
 #pragma unroll
@@ -287,7 +301,7 @@ __global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) 
                 }
                 acc[e] = a;
             }
-            __builtin_nontemporal_store(pack_words<T, kNW2>(acc), reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s2[q]) + (int64_t)o * p.s2_stride + o2));
+            __builtin_nontemporal_store(pack_elems<T>(acc), reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s2[q]) + (int64_t)o * p.s2_stride + o2));
         }
     }
 }
@@ -395,26 +409,27 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
 // quarter sizes here.
 template <class T>
 __device__ __forceinline__ float round16(float x) {
-    if constexpr (__is_same(T, bf16_t)) return bf16lo(pack_bf16(x, 0.f));
+    if constexpr (__is_same(T, float)) return x;
+    else if constexpr (__is_same(T, bf16_t)) return bf16lo(pack_bf16(x, 0.f));
     else return (float)as_f16x2(pack_f16(x, 0.f))[0];
 }
 
 template <class T, int ALGO2>
 __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Params p) {
-    typedef typename WordVec<kNW2>::type vec_t;
-    constexpr int E = kEPT2;
+    typedef typename ElemVec<T>::type vec_t;
+    constexpr int E = kEPT2, ES = (int)sizeof(T) == 4 ? 4 : 2;
     const int nq = p.Nh / E;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.Mh * nq) return;
     const int i = (int)(idx / nq), j = (int)(idx % nq) * E;
-    const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)i * p.Nh + j) * 2;
+    const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)i * p.Nh + j) * ES;
     float acc[4][4][E];   // [quadrant of C][quarter block within it][element]
     // second level of first-level product pp -> m[quarter block][element], rounded to T
     auto second = [&](int pp, float (&m)[4][E]) {
         float x[7][E];
 #pragma unroll
         for (int k = 0; k < 7; ++k)
-            unpack_words<T, kNW2>(__builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + (int64_t)(7 * pp + k) * p.p_ps * 2)), x[k]);
+            unpack_elems<T>(__builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + (int64_t)(7 * pp + k) * p.p_ps * ES)), x[k]);
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             if constexpr (ALGO2 == STHIP_STRASSEN) {
@@ -463,7 +478,7 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t row = (int64_t)(q >> 1) * mh + (b >> 1) * p.Mh + i, col = (int64_t)(q & 1) * nh + (b & 1) * p.Nh + j;
-            if (p.out_f32) {
+            if (p.out_f32 || ES == 4) {
                 float* d = reinterpret_cast<float*>(p.C) + row * p.c_rs + col;
 #pragma unroll
                 for (int e = 0; e < E; e += 4) {
@@ -472,15 +487,15 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
                     if (p.accumulate) o += *dd;
                     *dd = o;
                 }
-            } else {
+            } else if constexpr (ES == 2) {
                 vec_t* d = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.C) + (row * p.c_rs + col) * 2);
                 if (p.accumulate) {
                     float old[E];
-                    unpack_words<T, kNW2>(*d, old);
+                    unpack_elems<T>(*d, old);
 #pragma unroll
                     for (int e = 0; e < E; ++e) acc[q][b][e] += old[e];
                 }
-                __builtin_nontemporal_store(pack_words<T, kNW2>(acc[q][b]), d);
+                __builtin_nontemporal_store(pack_elems<T>(acc[q][b]), d);
             }
         }
 }
@@ -976,11 +991,11 @@ static int launch_recombine16(int dt, int algo, const void* prod, int64_t p_ps, 
 // S1 / S2 are laid out as the two-pass form lays them out (S1: five dense half-size sums s1_b
 // bytes apart; S2: for first-level operand p the sums at S2 + (5 p + o) * s2_b).
 static int64_t fill_combo2(Combo2Params& cp, View X, int64_t rq, int64_t cq, char* S1, size_t s1_b, char* S2, size_t s2_b,
-                           int side, int algo2) {
+                           int side, int algo2, int es = 2) {
     memset(&cp, 0, sizeof(cp));
     const bool row_major = X.cs == 1;
     for (int R = 0; R < 4; ++R)
-        for (int C = 0; C < 4; ++C) cp.x[4 * R + C] = X.p + ((int64_t)R * rq * X.rs + (int64_t)C * cq * X.cs) * 2;
+        for (int C = 0; C < 4; ++C) cp.x[4 * R + C] = X.p + ((int64_t)R * rq * X.rs + (int64_t)C * cq * X.cs) * es;
     // first-level operands in kernel order (level_operands): A side A11 S9 S2 S7 S5 S3 A22 with the
     // sums numbered as the outputs of kStrA (S2 S3 S5 S7 S9 = 0..4); B side S1 S10 B22 S8 S6 B11 S4
     // (kStrB: S1 S4 S6 S8 S10 = 0..4)
@@ -1147,8 +1162,9 @@ static int launch_recombine32(int algo, const void* prod, int64_t p_ps, char* C,
     return check_launch("recombine32");
 }
 
-// Two levels of fp32 operands as five launches (sums 1, sums 2, one grouped GEMM of the 49
-// products, 49 -> 7, 7 -> C; two Strassen levels, nothing rounded): worth it when
+// Two levels of fp32 operands in the same three-launch form (two Strassen levels, nothing
+// rounded; stage-mask bits 4 and 5 off: the five launches sums 1, sums 2, GEMM, 49 -> 7, 7 -> C,
+// which give the same bits): worth it when
 // the 49 quarter-size products fill the chip with 256 x 256 tiles, because the seven children
 // of the host recursion would each run their own seven products with a partly empty last round.
 static size_t two_level_f32_bytes(int64_t mh, int64_t nh, int64_t kh) {
@@ -1176,7 +1192,16 @@ static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh,
     char* P = SB2 + 35 * sb2;
     char* Mp = P + 49 * pb;
     const bool b_kc = B.rs == 1;
-    {
+    const bool fused = (g_stages & 32) != 0;   // sums of both levels in one pass, as for 16-bit operands
+    if (fused) {
+        Combo2Pair pp;
+        const int64_t na = fill_combo2(pp.side[0], A, mq, kq, SA1, sa1, SA2, sa2, 0, STHIP_STRASSEN, 4);
+        const int64_t nb = fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, STHIP_STRASSEN, 4);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        hipLaunchKernelGGL(quad_combos2_kernel<float>, grid, dim3(256), 0, stream, pp);
+        int rc = check_launch("quad_combos2 (fp32)");
+        if (rc) return rc;
+    } else {
         ComboPair pp;
         const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA, 4);
         const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB, 4);
@@ -1187,7 +1212,7 @@ static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh,
     }
     View xa1[7], xb1[7];
     level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1, 4);
-    {
+    if (!fused) {
         ComboMany pm;
         int64_t most = 0;
         for (int p = 0; p < 7; ++p) {
@@ -1214,6 +1239,14 @@ static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh,
     g.out_f32 = 1; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
     hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, stream);
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    if (g_stages & 16) {   // 49 -> C in one pass
+        Recombine16Params rp;
+        rp.prod = P; rp.p_ps = (int64_t)(pb / 4); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
+        rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = 1;
+        dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
+        hipLaunchKernelGGL((recombine16x2_kernel<float, STHIP_STRASSEN>), grid, dim3(256), 0, stream, rp);
+        return check_launch("recombine x2 (fp32)");
+    }
     int rc = launch_recombine32(STHIP_STRASSEN, P, (int64_t)(pb / 4), Mp, nh, (int64_t)(mb / 4), 7, mq, nq, false, stream);
     if (rc) return rc;
     return launch_recombine32(STHIP_STRASSEN, Mp, (int64_t)(mb / 4), C, c_rs, 0, 1, mh, nh, accumulate, stream);

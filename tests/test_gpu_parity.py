@@ -439,3 +439,25 @@ def test_fp32_large_tile_gaussian(hip):
     err = float(torch.linalg.norm(C - want) / torch.linalg.norm(want))
     print(f"fp32 4096^3 one level: rel_fro vs fp64 {err:.3e}")
     assert err <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("tb", [False, True])
+def test_fp32_two_levels_fused_passes_bit_identical(hip, tb):
+    """Two fp32 levels on the 49-product form: the one-pass sums and the one-pass recombination
+    add in the same order as the separate passes (stage-mask bits 4 and 5 off), so the results
+    are the same bits, and both are inside the fp32 tolerance against fp64."""
+    from strassen_hip import _capi
+    M, N, K = 4096, 4096, 512
+    A, B = _gauss((M, K), 91, 1.0, torch.float32), _gauss((K, N), 92, 1.0, torch.float32)
+    Ag, Bg = A.cuda(), _layout(B, tb)
+    fused = hip.gemm(Ag, Bg, algo="strassen", levels=2)
+    lib = _capi.load()
+    prev = lib.sthip_debug_set_stages(15)
+    try:
+        separate = hip.gemm(Ag, Bg, algo="strassen", levels=2)
+    finally:
+        lib.sthip_debug_set_stages(prev)
+    assert torch.equal(fused, separate)
+    want = A.double() @ B.double()
+    err = float(torch.linalg.norm(fused.cpu().double() - want) / torch.linalg.norm(want))
+    assert err <= TOL[torch.float32]
