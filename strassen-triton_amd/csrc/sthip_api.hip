@@ -139,7 +139,7 @@ __device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
             if constexpr (__is_same(T, bf16_t)) w[i] = pack_bf16(s[2 * i], s[2 * i + 1]);
             else w[i] = pack_f16(s[2 * i], s[2 * i + 1]);
         }
-        *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.out[o]) + out_off) = w;
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.out[o]) + out_off));
     }
 }
 
