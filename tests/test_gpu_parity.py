@@ -383,6 +383,12 @@ def test_every_pipelined_tile_exact(hip, monkeypatch, tile, dtype, algo, tb):
     assert torch.equal(Cacc.cpu().double(), C0.double() + want)
     Cn = hip.gemm(A[0, :, :128].contiguous().cuda(), _layout(B[0, :128], tb), algo=algo, levels=1)   # |C| <= 128: exact in 16 bit
     assert Cn.dtype == dtype and torch.equal(Cn.cpu().double(), A[0, :, :128].double() @ B[0, :128].double())
+    # the same in accumulate mode into a 16-bit C, two batch entries (|C| <= 128 + 3 stays exact)
+    A2, B2 = A[:, :, :128].contiguous(), B[:, :128].contiguous()
+    C16 = _ints((b, M, N), 54, -3, 3, dtype)
+    Cacc16 = C16.clone().cuda()
+    hip.gemm(A2.cuda(), _layout(B2, tb), out=Cacc16, algo=algo, levels=1, accumulate=True)
+    assert torch.equal(Cacc16.cpu().double(), C16.double() + A2.double() @ B2.double())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
