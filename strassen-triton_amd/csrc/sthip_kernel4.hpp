@@ -385,6 +385,32 @@ __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Para
     }
 }
 
+// The same for an fp32 result, in two halves of 64 rows (a wave's 128 x 64 fp32 tile is twice its
+// 16 KiB of LDS): row r of a half at r * 256, the 16-byte chunk c of a row at (c ^ (r % 16)) * 16.
+// Every store instruction then writes four rows x 256 contiguous bytes.
+__device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2Params& P, char* Cb, char* smem,
+                                                    int wave, int row, int col) {
+    const int lane = threadIdx.x & 63;
+    const int l16 = lane & 15, q = lane >> 4;
+    char* w = smem + wave * 16384;
+    float* dst = reinterpret_cast<float*>(Cb) + (int64_t)(row + q) * P.c_rs + (col + 4 * l16);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<f32x4*>(w + (16 * ii + l16) * 256 + (((4 * j + q) ^ l16) * 16)) = acc.t[4 * h + ii][j];
+        // read back: lane -> row 4 r + lane / 16 of the half, chunk lane % 16; same wave, LDS keeps order
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int rl = 4 * r + q;
+            const f32x4 v = *reinterpret_cast<const f32x4*>(w + rl * 256 + ((l16 ^ (rl & 15)) * 16));
+            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + (int64_t)(64 * h + 4 * r) * P.c_rs));
+        }
+    }
+}
+
 template <class T, bool B_KC>
 __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -422,6 +448,9 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     if (P.c_wide && !P.out_f32 && !P.accumulate && !(STHIP_DBG & 32)) {
         __syncthreads();   // every wave has read its last fragments: the stage buffers are free
         store_tile4_lds<T>(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
+    } else if (P.out_f32 && !P.accumulate && !(STHIP_DBG & 32)) {
+        __syncthreads();
+        store_tile4_lds_f32(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
     } else {
         store_tile4<T>(r, P, Cb, 0, tile_m + pipe.wm, tile_n + pipe.wn);
     }
