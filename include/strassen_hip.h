@@ -108,7 +108,10 @@ int sthip_run_accumulate(const void* A, const void* B, void* C,
 
 /* y[rows x D] = x[rows x D] x W^T (+ bias), W is D x D row-major, rows <= D.  The reference
  * pads x with zero rows up to D x D and slices afterwards (model/layers.py:246-274); here
- * the missing rows are simply never loaded or stored.  bias may be NULL. */
+ * the missing rows are simply never loaded or stored.  bias may be NULL; it is added to the
+ * rounded product and the sum rounded again, as the reference's `+ bias` does -- inside the
+ * recombination pass where the call runs as sums / grouped products / recombination, else by
+ * a pass of its own. */
 int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias, void* y,
                                   int64_t rows, int64_t D, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream);

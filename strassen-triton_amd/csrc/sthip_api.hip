@@ -338,8 +338,28 @@ struct Recombine16Params {
     int64_t p_ps;
     int Mh, Nh, accumulate;
     int out_f32;          // C is fp32 (no final rounding) instead of the operand type
+    const void* bias = nullptr;   // 16-bit, non-accumulating results: bias[column] is added to the rounded
+                                  // result and the sum rounded again, as a separate add would (model/layers.py:271-272)
 };
 
+// Bias of the Linear forward in flight on this thread: the recombination pass that writes `target`
+// adds it, so that no separate pass over the output is needed.
+struct BiasEpilogue { const void* bias = nullptr; const void* target = nullptr; bool applied = false; };
+static thread_local BiasEpilogue g_bias;
+static const void* take_bias(const void* C, bool accumulate, bool out_f32) {
+    if (!g_bias.bias || C != g_bias.target || accumulate || out_f32) return nullptr;
+    g_bias.applied = true;
+    return g_bias.bias;
+}
+
+
+// x rounded to T, as a float.
+template <class T>
+__device__ __forceinline__ float round16(float x) {
+    if constexpr (__is_same(T, float)) return x;
+    else if constexpr (__is_same(T, bf16_t)) return bf16lo(pack_bf16(x, 0.f));
+    else return (float)as_f16x2(pack_f16(x, 0.f))[0];
+}
 
 template <class T, int ALGO>
 __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Params p) {
@@ -388,6 +408,11 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
             unpack8<T>(*d, old);
 #pragma unroll
             for (int e = 0; e < 8; ++e) out[q][e] += old[e];
+        } else if (p.bias) {
+            float bv[8];
+            unpack8<T>(*reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.bias) + (int64_t)(j + (q & 1) * p.Nh) * 2), bv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[q][e] = round16<T>(out[q][e]) + bv[e];
         }
         u32x4 w;
 #pragma unroll
@@ -407,12 +432,6 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
 // order), so the result is bit-identical to the two passes -- without writing and re-reading the
 // seven half-size products.  One thread per 16-byte chunk of a quarter-size row; Mh, Nh are the
 // quarter sizes here.
-template <class T>
-__device__ __forceinline__ float round16(float x) {
-    if constexpr (__is_same(T, float)) return x;
-    else if constexpr (__is_same(T, bf16_t)) return bf16lo(pack_bf16(x, 0.f));
-    else return (float)as_f16x2(pack_f16(x, 0.f))[0];
-}
 
 template <class T, int ALGO2>
 __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Params p) {
@@ -494,6 +513,11 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
                     unpack_elems<T>(*d, old);
 #pragma unroll
                     for (int e = 0; e < E; ++e) acc[q][b][e] += old[e];
+                } else if (p.bias) {
+                    float bv[E];
+                    unpack_elems<T>(*reinterpret_cast<const vec_t*>(reinterpret_cast<const char*>(p.bias) + col * 2), bv);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[q][b][e] = round16<T>(acc[q][b][e]) + bv[e];
                 }
                 __builtin_nontemporal_store(pack_elems<T>(acc[q][b]), d);
             }
@@ -666,6 +690,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
         rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0; rp.p_ps = Mh * Nh; rp.out_f32 = out_f32 ? 1 : 0;
+        if (batch == 1 && (g_stages & 4)) rp.bias = take_bias(C, accumulate, out_f32);
         if (g_stages & 2) {
             p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
             p.out_f32 = out_f32 ? 1 : 0; p.accumulate = 0; p.nprod = 7;
@@ -1142,6 +1167,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     Recombine16Params rp;
     rp.prod = P; rp.p_ps = (int64_t)(pb / 2); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
     rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = out_f32 ? 1 : 0;
+    rp.bias = take_bias(C, accumulate, out_f32);
     dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
 #define GO(T, A) hipLaunchKernelGGL((recombine16x2_kernel<T, A>), grid, dim3(256), 0, stream, rp)
     if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
@@ -1600,10 +1626,14 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
     const int64_t Dp = round_up(D, q);
     View a = {reinterpret_cast<const char*>(x), D, 1};
     View b = {reinterpret_cast<const char*>(W), 1, D};   // W^T as a view
+    g_bias = BiasEpilogue{};
+    if (bias && dtype != STHIP_F32 && reinterpret_cast<uintptr_t>(bias) % 16 == 0) { g_bias.bias = bias; g_bias.target = y; }
     rc = multiply(a, b, reinterpret_cast<char*>(y), D, 1, rows, D, D, Dp, Dp, Dp, dtype, dtype, STHIP_STRASSEN, levels, false,
                   reinterpret_cast<char*>(workspace), workspace_bytes, s);
+    const bool bias_done = g_bias.applied;
+    g_bias = BiasEpilogue{};
     if (rc) return rc;
-    if (bias) {
+    if (bias && !bias_done) {
         const int64_t n = rows * D;
         const unsigned blocks = (unsigned)ceil_div(n, 256);
         char* yy = reinterpret_cast<char*>(y);

@@ -203,3 +203,31 @@ def test_cpu_tensors_are_refused():
     import fixed_strassen
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         fixed_strassen._strassen_base(torch.zeros(32, 32), torch.zeros(32, 32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("depth", [1, 2])
+def test_linear_strassen_bias_in_the_recombination_pass(dtype, depth):
+    """On tile-aligned 16-bit problems the bias is added by the recombination pass instead of a
+    pass of its own; the result is rounded before and after the addition, exactly as
+    `strassen(x, W.T) + bias` rounds (reference model/layers.py:264-272), so it must equal the
+    product computed without bias plus the bias added by torch, bit for bit."""
+    import strassen_hip
+    from model.layers import LinearStrassen
+    D = 1024
+    g = torch.Generator().manual_seed(31)
+    lin = LinearStrassen(D, D, bias=True, dtype=dtype, depth=depth, device="cuda")
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(D, D, generator=g) * D ** -0.5).to(dtype))
+        lin.bias.copy_(torch.randn(D, generator=g).to(dtype))
+    x = torch.randn(D, D, generator=g).to(dtype).cuda()
+    with torch.no_grad():
+        y = lin(x)
+        plain = strassen_hip.gemm(x, lin.weight.t(), levels=depth)
+        want = plain + lin.bias            # torch: fp32 add of two 16-bit values, rounded once
+    assert torch.equal(y, want)
+    # fewer rows than features: not the grouped path, the bias is added by the separate pass
+    with torch.no_grad():
+        y2 = lin(x[:300])
+    ref = x[:300].double() @ lin.weight.double().t() + lin.bias.double()
+    assert float(torch.linalg.norm(y2.double() - ref) / torch.linalg.norm(ref)) <= 2e-2
