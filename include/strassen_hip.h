@@ -116,6 +116,16 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
                                   int64_t rows, int64_t D, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* y[rows x out] = x[rows x in] x W^T (+ bias) for a Linear layer of any shape, W is out x in
+ * row-major, all tensors contiguous; bias as in sthip_linear_strassen_forward.  The reference's
+ * layer is square, a power of two and pads its input to D x D (model/layers.py:240, :255-262);
+ * this is the same forward with those constraints lifted (no padding: sizes that are not tile
+ * multiples take the kernels' edge tiles).  levels = 0 runs the classical product.
+ * Workspace as sthip_workspace_bytes(1, rows, out, in, dtype, dtype, STHIP_STRASSEN, levels). */
+int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y,
+                         int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* Description of the most recent failure on this thread ("" if none). */
 const char* sthip_last_error(void);
 

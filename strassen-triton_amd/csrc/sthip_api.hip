@@ -1646,6 +1646,34 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
     return STHIP_OK;
 }
 
+int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y,
+                         int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    g_err[0] = 0;
+    int rc = check_common(x, W, y, 1, rows, out_features, in_features, dtype, dtype, STHIP_STRASSEN, levels);
+    if (rc) return rc;
+    if (rows == 0 || out_features == 0) return STHIP_OK;
+    const int64_t sA[3] = {0, in_features, 1}, sB[3] = {0, 1, in_features}, sC[3] = {0, out_features, 1};   // B = W^T as a view
+    g_bias = BiasEpilogue{};
+    if (bias && dtype != STHIP_F32 && reinterpret_cast<uintptr_t>(bias) % 16 == 0) { g_bias.bias = bias; g_bias.target = y; }
+    rc = sthip_gemm(x, W, y, 1, rows, out_features, in_features, sA, sB, sC, dtype, dtype,
+                    levels > 0 ? STHIP_STRASSEN : STHIP_CLASSIC, levels, 0, workspace, workspace_bytes, stream);
+    const bool bias_done = g_bias.applied;
+    g_bias = BiasEpilogue{};
+    if (rc) return rc;
+    if (bias && !bias_done) {
+        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+        const unsigned blocks = (unsigned)ceil_div(rows * out_features, 256);
+        char* yy = reinterpret_cast<char*>(y);
+        const char* bb = reinterpret_cast<const char*>(bias);
+        if (dtype == STHIP_F32) hipLaunchKernelGGL(add_bias_kernel<float>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
+        else if (dtype == STHIP_F16) hipLaunchKernelGGL(add_bias_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
+        else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
+        return check_launch("add_bias");
+    }
+    return STHIP_OK;
+}
+
 int sthip_debug_set_stages(int mask) {
     const int old = g_stages;
     g_stages = mask & 63;

@@ -24,14 +24,15 @@ class LinearStrassen(_LinearStrassen):
 
 
 class _RectLinearFn(torch.autograd.Function):
-    """y = x W^T for any (rows, in) x (out, in): forward, dgrad dX = dY W and wgrad
-    dW = dY^T X are each one Strassen product over strided views, no padding, no copies."""
+    """y = x W^T + b for any (rows, in) x (out, in): forward, dgrad dX = dY W and wgrad
+    dW = dY^T X are each one Strassen product over strided views, no padding, no copies; the
+    bias is added by the forward product's recombination pass where it has one."""
 
     @staticmethod
-    def forward(ctx, x2d, weight, levels):
+    def forward(ctx, x2d, weight, bias, levels):
         ctx.save_for_backward(x2d, weight)
-        ctx.levels = levels
-        return strassen_hip.gemm(x2d, weight.t(), levels=levels)
+        ctx.levels, ctx.has_bias = levels, bias is not None
+        return strassen_hip.linear_forward_any(x2d, weight, bias, levels)
 
     @staticmethod
     def backward(ctx, dy):
@@ -39,7 +40,8 @@ class _RectLinearFn(torch.autograd.Function):
         dy = dy.contiguous()
         dx = strassen_hip.gemm(dy, weight, levels=ctx.levels) if ctx.needs_input_grad[0] else None
         dw = strassen_hip.gemm(dy.t(), x2d, levels=ctx.levels) if ctx.needs_input_grad[1] else None
-        return dx, dw, None
+        db = dy.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return dx, dw, db, None
 
 
 class LinearStrassenRect(nn.Linear):
@@ -57,9 +59,7 @@ class LinearStrassenRect(nn.Linear):
         *batch_dims, d_in = input.shape
         assert d_in == self.in_features, "Input dim mismatch"
         x2d = input.reshape(-1, d_in)
-        y = _RectLinearFn.apply(x2d, self.weight, max(1, int(self.depth)))
-        if self.bias is not None:
-            y = y + self.bias
+        y = _RectLinearFn.apply(x2d, self.weight, self.bias, max(1, int(self.depth)))
         return y.view(*batch_dims, self.out_features)
 
 

@@ -175,3 +175,24 @@ def linear_forward(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
         _capi.check(lib.sthip_linear_strassen_forward(x2d.data_ptr(), weight.data_ptr(), b_ptr, y.data_ptr(),
                                                       rows, D, dt, levels, ws_ptr, nbytes, _stream()))
     return y
+
+
+def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, levels: int) -> torch.Tensor:
+    """y = x2d @ weight.T (+ bias) for a weight of any shape (sthip_linear_forward): no padding,
+    the bias is added inside the recombination pass where the call takes the grouped path."""
+    _require_gpu(x2d, weight)
+    lib = _capi.load()
+    rows, d_in = x2d.shape
+    d_out = weight.shape[0]
+    if weight.shape[1] != d_in:
+        raise ValueError(f"shape mismatch: {tuple(x2d.shape)} @ {tuple(weight.shape)}^T")
+    x2d, weight = x2d.contiguous(), weight.contiguous()
+    dt = _dtype_code(x2d.dtype)
+    y = torch.empty((rows, d_out), dtype=x2d.dtype, device=x2d.device)
+    nbytes = lib.sthip_workspace_bytes(1, rows, d_out, d_in, dt, dt, ALGO_STRASSEN, levels)
+    ws, ws_ptr = _workspace(nbytes, x2d.device)
+    b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
+    with torch.cuda.device(x2d.device):
+        _capi.check(lib.sthip_linear_forward(x2d.data_ptr(), weight.data_ptr(), b_ptr, y.data_ptr(),
+                                             rows, d_in, d_out, dt, levels, ws_ptr, nbytes, _stream()))
+    return y

@@ -231,3 +231,26 @@ def test_linear_strassen_bias_in_the_recombination_pass(dtype, depth):
         y2 = lin(x[:300])
     ref = x[:300].double() @ lin.weight.double().t() + lin.bias.double()
     assert float(torch.linalg.norm(y2.double() - ref) / torch.linalg.norm(ref)) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_linear_strassen_rect_bias_in_the_recombination_pass(dtype):
+    """The non-square layer hands its bias to the forward product as well: same bits as the
+    product without bias plus torch's add, and the bias gradient is the column sum of dY."""
+    import strassen_hip
+    from model.layers import LinearStrassenRect
+    rows, d_in, d_out = 2048, 1024, 3072
+    g = torch.Generator().manual_seed(33)
+    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda")
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(d_out, d_in, generator=g) * d_in ** -0.5).to(dtype))
+        lin.bias.copy_(torch.randn(d_out, generator=g).to(dtype))
+    x = torch.randn(rows, d_in, generator=g).to(dtype).cuda().requires_grad_()
+    y = lin(x)
+    with torch.no_grad():
+        want = strassen_hip.gemm(x.detach(), lin.weight.t(), levels=1) + lin.bias
+    assert torch.equal(y.detach(), want)
+    dy = torch.randn(rows, d_out, generator=g).to(dtype).cuda()
+    y.backward(dy)
+    ref = dy.double().sum(0)
+    assert float(torch.linalg.norm(lin.bias.grad.double() - ref) / torch.linalg.norm(ref)) <= 2e-2
