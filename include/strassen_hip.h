@@ -126,6 +126,28 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
                          int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* A Linear layer whose weight stays put between calls (inference, or the reference's benchmark
+ * main_profiling.py:94-245, which times repeated forwards of one layer): the quadrant sums of
+ * W^T -- the five first-level sums, and for two levels the 35 second-level ones -- depend on W
+ * alone, so they can be formed once and kept in device memory; every forward then forms the
+ * input-side sums only.  The reference's LinearStrassen (model/layers.py:246-274) re-forms them
+ * on every call.  Results are bit-identical to sthip_linear_forward.
+ *
+ * sthip_linear_weight_sums_bytes: size of the buffer, or 0 where no sums can be kept (fp32,
+ * levels other than 1 or 2, halves -- quarters for two levels -- of in_features not a multiple of
+ * 64 or of out_features not a multiple of 128).
+ * sthip_linear_prepare_weight: forms the sums of W (out x in row-major, 16-byte aligned) into
+ * `sums` (256-byte aligned).  Call again whenever W's contents change.
+ * sthip_linear_forward_prepared: sthip_linear_forward reading those sums.  A call that does not
+ * take the sums / grouped products / recombination form (too few rows, odd rows) ignores them. */
+size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features, int dtype, int levels);
+int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_features, int dtype, int levels,
+                                void* sums, size_t sums_bytes, void* stream);
+int sthip_linear_forward_prepared(const void* x, const void* W, const void* sums, size_t sums_bytes,
+                                  const void* bias, void* y,
+                                  int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* Description of the most recent failure on this thread ("" if none). */
 const char* sthip_last_error(void);
 

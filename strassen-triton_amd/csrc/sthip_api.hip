@@ -352,6 +352,22 @@ static const void* take_bias(const void* C, bool accumulate, bool out_f32) {
     return g_bias.bias;
 }
 
+// Quadrant sums of a constant B operand formed ahead of the call (sthip_linear_prepare_weight).
+// The level -- or the two fused levels -- that find their B operand at `target` with the same
+// half extents read these and form the A-side sums only.  Layout: five first-level blocks of
+// kh x nh, then (two levels) 35 second-level blocks of kh/2 x nh/2, as in the workspace.
+struct PreparedSums {
+    const char* sums = nullptr; size_t bytes = 0; const void* target = nullptr;
+    int levels = 0; int64_t kh = 0, nh = 0; bool used = false;
+};
+static thread_local PreparedSums g_prep;
+static const char* take_prepared(const void* B, int levels, int64_t kh, int64_t nh, size_t need) {
+    if (!g_prep.sums || B != g_prep.target || levels != g_prep.levels || kh != g_prep.kh || nh != g_prep.nh ||
+        g_prep.bytes < need) return nullptr;
+    g_prep.used = true;
+    return g_prep.sums;
+}
+
 
 // x rounded to T, as a float.
 template <class T>
@@ -590,6 +606,8 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2);
         char* SA = ws;                                // [5][batch] blocks of Mh x Kh (storage order of A)
         char* SB = ws + (size_t)batch * 5 * sa_b;
+        const char* ready = algo == STHIP_STRASSEN && batch == 1 && b_kc ? take_prepared(B.p, 1, Kh, Nh, 5 * sb_b) : nullptr;
+        if (ready) SB = const_cast<char*>(ready);     // B-side sums formed ahead of the call: read, never written
         // region after the sums: parked fp32 tiles (256 x 128 kernel) or the seven 16-bit products (grouped paths)
         p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
@@ -598,7 +616,8 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             ComboPair pp;
             memset(&pp, 0, sizeof(pp));
             int64_t most = 0;
-            for (int side = 0; side < 2; ++side) {
+            const int sides = ready ? 1 : 2;
+            for (int side = 0; side < sides; ++side) {
                 ComboParams& cp = pp.side[side];
                 const int64_t r_ext = side == 0 ? (a_kc ? Mh : Kh) : (b_kc ? Nh : Kh);
                 const int64_t c_ext = side == 0 ? (a_kc ? Kh : Mh) : (b_kc ? Kh : Nh);
@@ -616,7 +635,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
                 cp.nout = nout; cp.rows = (int)r_ext; cp.chunks_per_row = (int)(c_ext / 8);
                 most = std::max(most, r_ext * (c_ext / 8));
             }
-            dim3 grid((unsigned)ceil_div(most, 256), (unsigned)batch, 2);
+            dim3 grid((unsigned)ceil_div(most, 256), (unsigned)batch, (unsigned)sides);
             if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
             else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
             int rc = check_launch("quad_combos");
@@ -1084,13 +1103,16 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     char* Mp = P + 49 * pb;
     const bool a_kc = A.cs == 1, b_kc = B.rs == 1;
     const int nout2 = algo == STHIP_STRASSEN ? 5 : 4;
+    // B-side sums of both levels formed ahead of the call: read, never written
+    const char* ready = algo == STHIP_STRASSEN && b_kc && (g_stages & 32) ? take_prepared(B.p, 2, kh, nh, 5 * sb1 + 35 * sb2) : nullptr;
+    if (ready) { SB1 = const_cast<char*>(ready); SB2 = SB1 + 5 * sb1; }
 
     // sums of both levels in one pass (bit 5 of the stage mask off: as two passes)
     if ((g_stages & 32) && (g_stages & 1)) {
         Combo2Pair pp;
         const int64_t na = fill_combo2(pp.side[0], A, mq, kq, SA1, sa1, SA2, sa2, 0, algo);
-        const int64_t nb = fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, algo);
-        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
+        const int64_t nb = ready ? 0 : fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, algo);
+        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, ready ? 1 : 2);
         if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
         else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
         int rc = check_launch("quad_combos2");
@@ -1672,6 +1694,67 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
         return check_launch("add_bias");
     }
     return STHIP_OK;
+}
+
+// Half extents of W^T (in_features x out_features) for which the weight-side sums can be formed
+// ahead of the call: 16-bit operands, one or two levels, halves (quarters) that the grouped paths take.
+static bool weight_sums_shape(int64_t in_features, int64_t out_features, int dtype, int levels) {
+    if (dtype != STHIP_BF16 && dtype != STHIP_F16) return false;
+    if (levels != 1 && levels != 2) return false;
+    const int64_t q = (int64_t)1 << levels;
+    if (in_features <= 0 || out_features <= 0 || in_features % q || out_features % q) return false;
+    return fast_shape(dtype, 128, out_features / q, in_features / q);
+}
+
+size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features, int dtype, int levels) {
+    if (!weight_sums_shape(in_features, out_features, dtype, levels)) return 0;
+    const int64_t kh = in_features / 2, nh = out_features / 2;
+    size_t n = 5 * align256(kh * nh * 2);
+    if (levels == 2) n += 35 * align256((kh / 2) * (nh / 2) * 2);
+    return n;
+}
+
+int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_features, int dtype, int levels,
+                                void* sums, size_t sums_bytes, void* stream) {
+    g_err[0] = 0;
+    const size_t need = sthip_linear_weight_sums_bytes(in_features, out_features, dtype, levels);
+    if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d (16-bit, 1 or 2 levels, aligned halves)",
+                           (long long)in_features, (long long)out_features, dtype, levels);
+    if (!W || !sums) return fail(STHIP_ERR_ARG, "null pointer");
+    if (!aligned_to(W, 16)) return fail(STHIP_ERR_ARG, "W must be 16-byte aligned");
+    if (!aligned_to(sums, 256)) return fail(STHIP_ERR_ARG, "the sums buffer must be 256-byte aligned");
+    if (sums_bytes < need) return fail(STHIP_ERR_WORKSPACE, "sums buffer too small: %zu < %zu bytes", sums_bytes, need);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const View B = {reinterpret_cast<const char*>(W), 1, in_features};   // W^T as a view
+    const int64_t kh = in_features / 2, nh = out_features / 2;
+    const size_t sb1 = align256(kh * nh * 2);
+    char* S1 = reinterpret_cast<char*>(sums);
+    if (levels == 1) return run_combos(dtype, B, kh, nh, S1, sb1, 5, kStrB, s);
+    const size_t sb2 = align256((kh / 2) * (nh / 2) * 2);
+    Combo2Pair pp;
+    memset(&pp, 0, sizeof(pp));
+    const int64_t nb = fill_combo2(pp.side[0], B, kh / 2, nh / 2, S1, sb1, S1 + 5 * sb1, sb2, 1, STHIP_STRASSEN);
+    dim3 grid((unsigned)ceil_div(nb, 256), 1, 1);
+    if (dtype == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, s, pp);
+    else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, s, pp);
+    return check_launch("quad_combos2 (weight)");
+}
+
+int sthip_linear_forward_prepared(const void* x, const void* W, const void* sums, size_t sums_bytes, const void* bias, void* y,
+                                  int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    g_err[0] = 0;
+    const size_t need = sthip_linear_weight_sums_bytes(in_features, out_features, dtype, levels);
+    if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d",
+                           (long long)in_features, (long long)out_features, dtype, levels);
+    if (!sums || !aligned_to(sums, 256)) return fail(STHIP_ERR_ARG, "the sums buffer must be non-null and 256-byte aligned");
+    if (sums_bytes < need) return fail(STHIP_ERR_WORKSPACE, "sums buffer too small: %zu < %zu bytes", sums_bytes, need);
+    g_prep = PreparedSums{};
+    g_prep.sums = reinterpret_cast<const char*>(sums); g_prep.bytes = sums_bytes; g_prep.target = W;
+    g_prep.levels = levels; g_prep.kh = in_features / 2; g_prep.nh = out_features / 2;
+    const int rc = sthip_linear_forward(x, W, bias, y, rows, in_features, out_features, dtype, levels, workspace, workspace_bytes, stream);
+    g_prep = PreparedSums{};
+    return rc;
 }
 
 int sthip_debug_set_stages(int mask) {

@@ -46,9 +46,11 @@ class _LinearFn(torch.autograd.Function):
     dW = dY^T X are Strassen products over views of the saved tensors."""
 
     @staticmethod
-    def forward(ctx, x2d, weight, bias, levels):
+    def forward(ctx, x2d, weight, bias, levels, weight_sums=None):
         ctx.save_for_backward(x2d, weight)
         ctx.levels, ctx.has_bias = levels, bias is not None
+        if weight_sums is not None:
+            return strassen_hip.linear_forward_any(x2d, weight, bias, levels, weight_sums)
         return strassen_hip.linear_forward(x2d, weight, bias, levels)
 
     @staticmethod
@@ -58,19 +60,27 @@ class _LinearFn(torch.autograd.Function):
         dx = strassen_hip.gemm(dy, weight, levels=1) if ctx.needs_input_grad[0] else None
         dw = strassen_hip.gemm(dy.t(), x2d, levels=1) if ctx.needs_input_grad[1] else None
         db = dy.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
-        return dx, dw, db, None
+        return dx, dw, db, None, None
 
 
 class LinearStrassen(nn.Linear):
     """nn.Linear whose matmul is the Strassen kernel (reference fixed_strassen.py:128-169,
-    model/layers.py:232-274): square power-of-two features, at most D input rows."""
+    model/layers.py:232-274): square power-of-two features, at most D input rows.
+
+    cache_weight_sums (not in the reference, off by default): keep the quadrant sums of the
+    weight in device memory between calls (1.25 x the weight's bytes at depth 1, 2.2 x at
+    depth 2) instead of forming them in every forward; for 16-bit weights, D x D inputs and one
+    or two levels, same bits.  The sums follow the weight's version counter: after a write that
+    bypasses it (through .data) call weight_sums.clear()."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=torch.float32,
-                 depth: int = 1, device: str = "cuda") -> None:
+                 depth: int = 1, device: str = "cuda", cache_weight_sums: bool = False) -> None:
         assert in_features == out_features and (log2(in_features)).is_integer(), \
             "Transform must be square and a power of 2"
         super().__init__(in_features, out_features, bias, device, dtype)
         self.depth = depth
+        self.cache_weight_sums = cache_weight_sums
+        self.weight_sums = strassen_hip.WeightSums()
 
     def forward(self, input: Tensor):
         *batch_dims, D_in = input.shape
@@ -82,5 +92,6 @@ class LinearStrassen(nn.Linear):
                 f"Input M ({M}) > D ({D}). Cannot pad input to DxD. "
                 f"You MUST use the method that pads BOTH input and weights to PxP.")
         levels = max(1, practical_levels(D, reference_levels(D, self.depth)))
-        out = _LinearFn.apply(input.reshape(M, D), self.weight, self.bias, levels)
+        sums = self.weight_sums.get(self.weight, levels) if self.cache_weight_sums and M == D and levels <= 2 else None
+        out = _LinearFn.apply(input.reshape(M, D), self.weight, self.bias, levels, sums)
         return out.view(*batch_dims, D)

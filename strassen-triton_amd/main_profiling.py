@@ -11,6 +11,7 @@ stream, and the grid is limited by --max-n.
     python main_profiling.py [--dtype bf16|fp16|fp32] [--max-n 16384] [--min-n 1024]
     python main_profiling.py --gpt2      # the Linear shapes of GPT-2 small, forward and backward
     python main_profiling.py --json out.json   # also write the rows as JSON
+    python main_profiling.py --cache-weight-sums   # LinearStrassen keeps the weight's quadrant sums between calls
 """
 from __future__ import annotations
 
@@ -65,13 +66,15 @@ def _bench(fn, warmup: int, runs: int, flush: torch.Tensor) -> list[float]:
 @torch.no_grad()
 def benchmark_linear_layers(N_dim: int, strassen_depth: int, use_bias: bool = False,
                             dtype=torch.bfloat16, device: str = "cuda",
-                            num_warmup: int = 10, num_runs: int = 50, flush=None) -> dict:
+                            num_warmup: int = 10, num_runs: int = 50, flush=None,
+                            cache_weight_sums: bool = False) -> dict:
     assert N_dim > 0 and (N_dim & (N_dim - 1)) == 0, "N_dim (features) must be a power of 2."
     res = {"N_dim": N_dim, "strassen_depth": strassen_depth, "bias": use_bias}
     x = torch.randn(N_dim, N_dim, device=device, dtype=dtype)
     std = nn.Linear(N_dim, N_dim, bias=use_bias, device=device, dtype=dtype).eval()
-    ours = LinearStrassen(N_dim, N_dim, bias=use_bias, dtype=dtype, depth=strassen_depth, device=device).eval()
-    ours.weight.data.copy_(std.weight.data)
+    ours = LinearStrassen(N_dim, N_dim, bias=use_bias, dtype=dtype, depth=strassen_depth, device=device,
+                          cache_weight_sums=cache_weight_sums).eval()
+    ours.weight.data.copy_(std.weight.data)   # before the first forward: writes through .data do not refresh kept sums
     if use_bias:
         ours.bias.data.copy_(std.bias.data)
 
@@ -103,7 +106,8 @@ def format_row(r: dict) -> str:
             f"{r['strassen_tflops']:>17.2f} | {r['max_abs_diff']:>12.3e} | {str(r['allclose']):>8s}")
 
 
-def profile_linear_layers(dtype=torch.bfloat16, min_n: int = 1024, max_n: int = 16384) -> list[dict]:
+def profile_linear_layers(dtype=torch.bfloat16, min_n: int = 1024, max_n: int = 16384,
+                          cache_weight_sums: bool = False) -> list[dict]:
     flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
     rows = []
     print(HEADER)
@@ -112,7 +116,8 @@ def profile_linear_layers(dtype=torch.bfloat16, min_n: int = 1024, max_n: int = 
         if n < min_n or n > max_n:
             continue
         warmup, runs = _runs_for(n)
-        r = benchmark_linear_layers(n, depth, dtype=dtype, num_warmup=warmup, num_runs=runs, flush=flush)
+        r = benchmark_linear_layers(n, depth, dtype=dtype, num_warmup=warmup, num_runs=runs, flush=flush,
+                                    cache_weight_sums=cache_weight_sums)
         rows.append(r)
         print(format_row(r), flush=True)
         torch.cuda.empty_cache()
@@ -161,6 +166,8 @@ if __name__ == "__main__":
     ap.add_argument("--min-n", type=int, default=1024)
     ap.add_argument("--max-n", type=int, default=16384)
     ap.add_argument("--gpt2", action="store_true", help="GPT-2-small Linear shapes instead of the square grid")
+    ap.add_argument("--cache-weight-sums", action="store_true",
+                    help="keep the quadrant sums of the weight between calls (16-bit, depth 1 and 2)")
     ap.add_argument("--json", default=None, help="write the measured rows to this file as JSON")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -169,7 +176,7 @@ if __name__ == "__main__":
     if args.gpt2:
         rows = profile_gpt2_linears(dtype=_DTYPES[args.dtype])
     else:
-        rows = profile_linear_layers(_DTYPES[args.dtype], args.min_n, args.max_n)
+        rows = profile_linear_layers(_DTYPES[args.dtype], args.min_n, args.max_n, args.cache_weight_sums)
     if args.json:
         with open(args.json, "w") as f:
             json.dump({"device": torch.cuda.get_device_name(0), "dtype": args.dtype, "rows": rows}, f, indent=1)

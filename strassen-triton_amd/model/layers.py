@@ -18,8 +18,8 @@ class LinearStrassen(_LinearStrassen):
     model/layers.py:232-244 (dtype defaults to None; depth 2 selects the two-layer product)."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=None,
-                 depth: int = 1, device: str = "cuda") -> None:
-        super().__init__(in_features, out_features, bias, dtype, depth, device)
+                 depth: int = 1, device: str = "cuda", cache_weight_sums: bool = False) -> None:
+        super().__init__(in_features, out_features, bias, dtype, depth, device, cache_weight_sums)
         self.strassen_func = strassen_matmul_two_layers if depth == 2 else _strassen_base
 
 
@@ -29,10 +29,10 @@ class _RectLinearFn(torch.autograd.Function):
     bias is added by the forward product's recombination pass where it has one."""
 
     @staticmethod
-    def forward(ctx, x2d, weight, bias, levels):
+    def forward(ctx, x2d, weight, bias, levels, weight_sums=None):
         ctx.save_for_backward(x2d, weight)
         ctx.levels, ctx.has_bias = levels, bias is not None
-        return strassen_hip.linear_forward_any(x2d, weight, bias, levels)
+        return strassen_hip.linear_forward_any(x2d, weight, bias, levels, weight_sums)
 
     @staticmethod
     def backward(ctx, dy):
@@ -41,25 +41,30 @@ class _RectLinearFn(torch.autograd.Function):
         dx = strassen_hip.gemm(dy, weight, levels=ctx.levels) if ctx.needs_input_grad[0] else None
         dw = strassen_hip.gemm(dy.t(), x2d, levels=ctx.levels) if ctx.needs_input_grad[1] else None
         db = dy.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
-        return dx, dw, db, None
+        return dx, dw, db, None, None
 
 
 class LinearStrassenRect(nn.Linear):
     """nn.Linear of any shape whose three GEMMs are Strassen products.  Lifts the constraints
     of the reference's layer (model/layers.py:240, :255-262: square, power of two, at most D
     input rows, input padded to D x D): sizes that are odd or not tile multiples are handled
-    by the kernels' zero-padding edge tiles, so nothing is padded or sliced in memory."""
+    by the kernels' zero-padding edge tiles, so nothing is padded or sliced in memory.
+    cache_weight_sums: as for LinearStrassen; shapes for which no sums are kept run as before."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=None,
-                 depth: int = 1, device: str = "cuda") -> None:
+                 depth: int = 1, device: str = "cuda", cache_weight_sums: bool = False) -> None:
         super().__init__(in_features, out_features, bias, device, dtype)
         self.depth = depth
+        self.cache_weight_sums = cache_weight_sums
+        self.weight_sums = strassen_hip.WeightSums()
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         *batch_dims, d_in = input.shape
         assert d_in == self.in_features, "Input dim mismatch"
         x2d = input.reshape(-1, d_in)
-        y = _RectLinearFn.apply(x2d, self.weight, self.bias, max(1, int(self.depth)))
+        levels = max(1, int(self.depth))
+        sums = self.weight_sums.get(self.weight, levels) if self.cache_weight_sums and levels <= 2 else None
+        y = _RectLinearFn.apply(x2d, self.weight, self.bias, levels, sums)
         return y.view(*batch_dims, self.out_features)
 
 

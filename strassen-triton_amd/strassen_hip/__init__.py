@@ -1,6 +1,7 @@
 """Host side of the MI355X Strassen library: tensors in, C-ABI calls out."""
-from .ops import (ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD, StrassenMatmul, gemm, linear_forward, linear_forward_any,
-                  matmul, run_accumulate, workspace_bytes)
+from .ops import (ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD, StrassenMatmul, WeightSums, gemm, linear_forward,
+                  linear_forward_any, matmul, prepare_weight, run_accumulate, workspace_bytes)
 
 __all__ = ["gemm", "matmul", "run_accumulate", "linear_forward", "linear_forward_any", "StrassenMatmul", "workspace_bytes",
+           "prepare_weight", "WeightSums",
            "ALGO_CLASSIC", "ALGO_STRASSEN", "ALGO_WINOGRAD"]

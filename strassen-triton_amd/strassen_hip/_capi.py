@@ -24,6 +24,9 @@ SIGNATURES = {
                                     _vp, _sz, _vp]),
     "sthip_linear_strassen_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp, _sz, _vp]),
     "sthip_linear_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "sthip_linear_weight_sums_bytes": (_sz, [_i64, _i64, _int, _int]),
+    "sthip_linear_prepare_weight": (_int, [_vp, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "sthip_linear_forward_prepared": (_int, [_vp, _vp, _vp, _sz, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
     "sthip_last_error": (ctypes.c_char_p, []),
     "sthip_version": (_int, []),
     "sthip_debug_transpose_read": (_int, [_vp, _vp]),

@@ -177,9 +177,12 @@ def linear_forward(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     return y
 
 
-def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, levels: int) -> torch.Tensor:
+def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, levels: int,
+                       weight_sums: torch.Tensor | None = None) -> torch.Tensor:
     """y = x2d @ weight.T (+ bias) for a weight of any shape (sthip_linear_forward): no padding,
-    the bias is added inside the recombination pass where the call takes the grouped path."""
+    the bias is added inside the recombination pass where the call takes the grouped path.
+    weight_sums: the buffer prepare_weight made for this weight and these levels; the call then
+    forms the input-side sums only (sthip_linear_forward_prepared), with the same bits."""
     _require_gpu(x2d, weight)
     lib = _capi.load()
     rows, d_in = x2d.shape
@@ -193,6 +196,52 @@ def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tens
     ws, ws_ptr = _workspace(nbytes, x2d.device)
     b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
     with torch.cuda.device(x2d.device):
-        _capi.check(lib.sthip_linear_forward(x2d.data_ptr(), weight.data_ptr(), b_ptr, y.data_ptr(),
-                                             rows, d_in, d_out, dt, levels, ws_ptr, nbytes, _stream()))
+        if weight_sums is not None:
+            _capi.check(lib.sthip_linear_forward_prepared(x2d.data_ptr(), weight.data_ptr(), weight_sums.data_ptr(),
+                                                          weight_sums.numel(), b_ptr, y.data_ptr(),
+                                                          rows, d_in, d_out, dt, levels, ws_ptr, nbytes, _stream()))
+        else:
+            _capi.check(lib.sthip_linear_forward(x2d.data_ptr(), weight.data_ptr(), b_ptr, y.data_ptr(),
+                                                 rows, d_in, d_out, dt, levels, ws_ptr, nbytes, _stream()))
     return y
+
+
+def prepare_weight(weight: torch.Tensor, levels: int) -> torch.Tensor | None:
+    """The quadrant sums of weight^T for `levels` Strassen levels as an opaque device buffer
+    (sthip_linear_prepare_weight), or None where the library keeps none for this shape and type.
+    Valid until the weight's contents change."""
+    _require_gpu(weight)
+    lib = _capi.load()
+    if weight.dim() != 2 or not weight.is_contiguous():
+        return None
+    d_out, d_in = weight.shape
+    if weight.dtype not in (torch.bfloat16, torch.float16):
+        return None
+    dt = _dtype_code(weight.dtype)
+    nbytes = lib.sthip_linear_weight_sums_bytes(d_in, d_out, dt, levels)
+    if nbytes == 0:
+        return None
+    sums = torch.empty(nbytes, dtype=torch.uint8, device=weight.device)
+    with torch.cuda.device(weight.device):
+        _capi.check(lib.sthip_linear_prepare_weight(weight.data_ptr(), d_in, d_out, dt, levels,
+                                                    sums.data_ptr(), nbytes, _stream()))
+    return sums
+
+
+class WeightSums:
+    """Keeps the prepared sums of one weight tensor and forms them again when the tensor is
+    written (its version counter moves), replaced, or asked for at another depth."""
+
+    def __init__(self) -> None:
+        self._key = None
+        self._sums = None
+
+    def get(self, weight: torch.Tensor, levels: int) -> torch.Tensor | None:
+        key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, levels)
+        if key != self._key:
+            self._sums = prepare_weight(weight, levels)
+            self._key = key
+        return self._sums
+
+    def clear(self) -> None:
+        self._key, self._sums = None, None

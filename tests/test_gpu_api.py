@@ -254,3 +254,77 @@ def test_linear_strassen_rect_bias_in_the_recombination_pass(dtype):
     y.backward(dy)
     ref = dy.double().sum(0)
     assert float(torch.linalg.norm(lin.bias.grad.double() - ref) / torch.linalg.norm(ref)) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("levels", [1, 2])
+@pytest.mark.parametrize("rows,d_in,d_out,bias", [(1024, 1024, 1024, False), (2048, 1536, 1024, True), (4096, 4096, 4096, True)])
+def test_prepared_weight_sums_same_bits(dtype, levels, rows, d_in, d_out, bias):
+    """The forward that reads weight-side sums formed ahead of the call gives the bits of the
+    forward that forms them itself -- and does read them: handed the sums of another weight it
+    gives another result."""
+    import strassen_hip
+    g = torch.Generator().manual_seed(rows + d_in + levels)
+    x = torch.randn(rows, d_in, generator=g).to(dtype).cuda()
+    w = (torch.randn(d_out, d_in, generator=g) * d_in ** -0.5).to(dtype).cuda()
+    b = torch.randn(d_out, generator=g).to(dtype).cuda() if bias else None
+    want = strassen_hip.linear_forward_any(x, w, b, levels)
+    sums = strassen_hip.prepare_weight(w, levels)
+    assert sums is not None
+    got = strassen_hip.linear_forward_any(x, w, b, levels, sums)
+    assert torch.equal(got, want)
+    again = strassen_hip.linear_forward_any(x, w, b, levels, sums)   # the sums are read, never written
+    assert torch.equal(again, want)
+    other = strassen_hip.prepare_weight(w.flip(0).contiguous(), levels)
+    assert not torch.equal(strassen_hip.linear_forward_any(x, w, b, levels, other), want)
+    ref = x.double() @ w.double().t() + (b.double() if bias else 0)
+    assert float(torch.linalg.norm(got.double() - ref) / torch.linalg.norm(ref)) <= 2e-2
+
+
+def test_prepared_weight_sums_where_none_are_kept():
+    import strassen_hip
+    assert strassen_hip.prepare_weight(torch.zeros(1024, 1024, device="cuda"), 1) is None                          # fp32
+    assert strassen_hip.prepare_weight(torch.zeros(1024, 1024, device="cuda", dtype=torch.bfloat16), 3) is None    # depth
+    assert strassen_hip.prepare_weight(torch.zeros(1000, 1000, device="cuda", dtype=torch.bfloat16), 1) is None    # shape
+    # too few rows for the grouped form: the sums are ignored, the result is the plain forward's
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(24, 1024, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(1024, 1024, generator=g) / 32).to(torch.bfloat16).cuda()
+    sums = strassen_hip.prepare_weight(w, 1)
+    assert torch.equal(strassen_hip.linear_forward_any(x, w, None, 1, sums), strassen_hip.linear_forward_any(x, w, None, 1))
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+def test_layers_keep_weight_sums_between_calls(depth):
+    """LinearStrassen and LinearStrassenRect with cache_weight_sums: same bits as without, the
+    sums are formed once per weight version and again after the weight is written."""
+    import strassen_hip
+    from model.layers import LinearStrassen, LinearStrassenRect
+    g = torch.Generator().manual_seed(8 + depth)
+    for make, rows, d_in, d_out in ((LinearStrassen, 2048, 2048, 2048), (LinearStrassenRect, 1024, 1024, 3072)):
+        plain = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda")
+        keep = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda", cache_weight_sums=True)
+        with torch.no_grad():
+            plain.weight.copy_((torch.randn(d_out, d_in, generator=g) * d_in ** -0.5).to(torch.bfloat16))
+            plain.bias.copy_(torch.randn(d_out, generator=g).to(torch.bfloat16))
+            keep.weight.copy_(plain.weight)
+            keep.bias.copy_(plain.bias)
+        x = torch.randn(rows, d_in, generator=g).to(torch.bfloat16).cuda()
+        with torch.no_grad():
+            assert torch.equal(keep(x), plain(x))
+            first = keep.weight_sums._sums
+            assert first is not None
+            assert torch.equal(keep(x), plain(x))
+            assert keep.weight_sums._sums is first          # not formed again
+            plain.weight.mul_(0.5)
+            keep.weight.mul_(0.5)
+            assert torch.equal(keep(x), plain(x))
+            assert keep.weight_sums._sums is not first      # the write moved the version counter
+        # training step through the caching layer: gradients as without the cache
+        xg = x.clone().requires_grad_()
+        xk = x.clone().requires_grad_()
+        dy = torch.randn(rows, d_out, generator=g).to(torch.bfloat16).cuda()
+        plain(xg).backward(dy)
+        keep(xk).backward(dy)
+        assert torch.equal(xg.grad, xk.grad) and torch.equal(plain.weight.grad, keep.weight.grad)
+        assert torch.equal(plain.bias.grad, keep.bias.grad)

@@ -87,6 +87,32 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4 + f32(256)
 
 
+def test_weight_sums_size_and_argument_errors():
+    """Sums of a constant weight: five half-size blocks for one level, 35 quarter-size ones more
+    for two; none for fp32, other depths or halves the grouped paths do not take.  Bad buffers are
+    refused before anything is launched."""
+    from strassen_hip import _capi
+    lib = _capi.load()
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 1) == 5 * 512 * 512 * 2
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 1, 2) == 5 * 512 * 512 * 2 + 35 * 256 * 256 * 2
+    assert lib.sthip_linear_weight_sums_bytes(768, 3072, 2, 1) == 5 * 384 * 1536 * 2
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 0, 1) == 0      # fp32
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 3) == 0      # three levels
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 0) == 0
+    assert lib.sthip_linear_weight_sums_bytes(1000, 1024, 2, 1) == 0      # 500 is no multiple of 64
+    assert lib.sthip_linear_weight_sums_bytes(1024, 768, 2, 2) == 0       # 192 is no multiple of 128
+    w, buf = ctypes.c_void_p(4096), ctypes.c_void_p(8192)
+    assert lib.sthip_linear_prepare_weight(w, 1024, 1024, 0, 1, buf, 1 << 30, None) == -1
+    assert b"no weight-side sums" in lib.sthip_last_error()
+    assert lib.sthip_linear_prepare_weight(w, 1024, 1024, 2, 1, buf, 100, None) == -4
+    assert b"too small" in lib.sthip_last_error()
+    assert lib.sthip_linear_prepare_weight(w, 1024, 1024, 2, 1, ctypes.c_void_p(8200), 1 << 30, None) == -5
+    assert lib.sthip_linear_prepare_weight(None, 1024, 1024, 2, 1, buf, 1 << 30, None) == -5
+    assert lib.sthip_linear_forward_prepared(w, w, buf, 100, None, w, 1024, 1024, 1024, 2, 1, None, 0, None) == -4
+    assert lib.sthip_linear_forward_prepared(w, w, None, 1 << 30, None, w, 1024, 1024, 1024, 2, 1, None, 0, None) == -5
+    assert lib.sthip_linear_forward_prepared(w, w, buf, 1 << 30, None, w, 1024, 1024, 1024, 0, 1, None, 0, None) == -1
+
+
 def test_reference_recursion_depth():
     from _levels import practical_levels, reference_levels
     # fixed_strassen.py:71-114 traced by hand
