@@ -62,6 +62,8 @@ def main() -> None:
     ap.add_argument("--tokens", type=int, default=8192, help="batch x sequence; sequences of 1024")
     ap.add_argument("--dtype", choices=sorted(_DTYPES), default="bf16")
     ap.add_argument("--backward", action="store_true", help="time forward + backward instead of forward only")
+    ap.add_argument("--cache-weight-sums", action="store_true",
+                    help="the replaced layers keep their weights' quadrant sums between calls (inference)")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: this demo needs an MI355X")
@@ -69,7 +71,8 @@ def main() -> None:
     torch.manual_seed(0)
     std = Block(args.dim, args.heads, dtype=dtype)
     ours = copy.deepcopy(std)
-    replace_linear_with_strassen(ours, min_size=128, depth=1, square_only=False)
+    replace_linear_with_strassen(ours, min_size=128, depth=1, square_only=False,
+                                 cache_weight_sums=args.cache_weight_sums)
     seq = min(1024, args.tokens)
     x = torch.randn(args.tokens // seq, seq, args.dim, device="cuda", dtype=dtype)
 

@@ -69,19 +69,21 @@ class LinearStrassenRect(nn.Linear):
 
 
 def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: int = 1,
-                                 square_only: bool = True):
+                                 square_only: bool = True, cache_weight_sums: bool = False):
     """Swap every square nn.Linear of at least min_size features for LinearStrassen, in
     place, keeping weights and bias (reference model/layers.py:279-300).  With
     square_only=False every layer whose smaller side is at least min_size becomes a
     LinearStrassenRect instead (any shape, any number of input rows -- the reference's layer
-    refuses more than D rows); below min_size a layer stays an nn.Linear, i.e. a classical GEMM."""
+    refuses more than D rows); below min_size a layer stays an nn.Linear, i.e. a classical GEMM.
+    cache_weight_sums is handed to the new layers."""
     for name, child in module.named_children():
         if isinstance(child, nn.Linear) and not isinstance(child, (_LinearStrassen, LinearStrassenRect)):
             if not square_only and min(child.in_features, child.out_features) >= min_size:
                 print(f"Replacing '{name}' with LinearStrassenRect.")
                 new_layer = LinearStrassenRect(child.in_features, child.out_features,
                                                bias=child.bias is not None, device=child.weight.device,
-                                               dtype=child.weight.dtype, depth=depth)
+                                               dtype=child.weight.dtype, depth=depth,
+                                           cache_weight_sums=cache_weight_sums)
                 new_layer.weight.data.copy_(child.weight.data)
                 if child.bias is not None:
                     new_layer.bias.data.copy_(child.bias.data)
@@ -90,7 +92,8 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
                 print(f"Replacing '{name}' with LinearStrassen.")
                 new_layer = LinearStrassen(child.in_features, child.out_features,
                                            bias=child.bias is not None, device=child.weight.device,
-                                           dtype=child.weight.dtype, depth=depth)
+                                           dtype=child.weight.dtype, depth=depth,
+                                           cache_weight_sums=cache_weight_sums)
                 new_layer.weight.data.copy_(child.weight.data)
                 if child.bias is not None:
                     new_layer.bias.data.copy_(child.bias.data)
@@ -98,4 +101,4 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
             else:
                 print(f"Skipping '{name}': Not square or too small.")
         elif len(list(child.children())) > 0:
-            replace_linear_with_strassen(child, min_size, depth, square_only)
+            replace_linear_with_strassen(child, min_size, depth, square_only, cache_weight_sums)
