@@ -6,6 +6,7 @@ kernels behind libstrassen_hip.so.  Tensors must live on the GPU: there is no CP
 from __future__ import annotations
 
 import ctypes
+import weakref
 
 import torch
 
@@ -233,15 +234,25 @@ class WeightSums:
     written (its version counter moves), replaced, or asked for at another depth."""
 
     def __init__(self) -> None:
-        self._key = None
-        self._sums = None
+        self.clear()
 
     def get(self, weight: torch.Tensor, levels: int) -> torch.Tensor | None:
         key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, levels)
-        if key != self._key:
+        same_tensor = self._owner is not None and self._owner() is weight
+        if not same_tensor or key != self._key:
             self._sums = prepare_weight(weight, levels)
-            self._key = key
+            self._key, self._owner = key, weakref.ref(weight)
         return self._sums
 
     def clear(self) -> None:
-        self._key, self._sums = None, None
+        self._key, self._sums, self._owner = None, None, None
+
+    # a copied or unpickled layer starts without sums and forms its own on first use
+    def __getstate__(self):
+        return {}
+
+    def __setstate__(self, state) -> None:
+        self.clear()
+
+    def __deepcopy__(self, memo):
+        return WeightSums()

@@ -320,6 +320,12 @@ def test_layers_keep_weight_sums_between_calls(depth):
             keep.weight.mul_(0.5)
             assert torch.equal(keep(x), plain(x))
             assert keep.weight_sums._sums is not first      # the write moved the version counter
+            import copy
+            twin = copy.deepcopy(keep)
+            assert twin.weight_sums._sums is None and torch.equal(twin(x), plain(x))
+            second = keep.weight_sums._sums
+            keep.weight = torch.nn.Parameter(plain.weight.detach().clone())   # another tensor object, same values
+            assert torch.equal(keep(x), plain(x)) and keep.weight_sums._sums is not second
         # training step through the caching layer: gradients as without the cache
         xg = x.clone().requires_grad_()
         xk = x.clone().requires_grad_()

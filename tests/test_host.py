@@ -113,6 +113,17 @@ def test_weight_sums_size_and_argument_errors():
     assert lib.sthip_linear_forward_prepared(w, w, buf, 1 << 30, None, w, 1024, 1024, 1024, 0, 1, None, 0, None) == -1
 
 
+def test_weight_sums_holder_survives_copy_and_pickle():
+    """A layer that keeps weight sums can be deep-copied and pickled: the copy starts empty."""
+    import copy
+    import pickle
+    import strassen_hip
+    held = strassen_hip.WeightSums()
+    held._key, held._sums = ("stale",), object()
+    for twin in (copy.deepcopy(held), pickle.loads(pickle.dumps(held))):
+        assert twin._key is None and twin._sums is None and twin._owner is None
+
+
 def test_reference_recursion_depth():
     from _levels import practical_levels, reference_levels
     # fixed_strassen.py:71-114 traced by hand
