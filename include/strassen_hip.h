@@ -128,14 +128,15 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
 
 /* A Linear layer whose weight stays put between calls (inference, or the reference's benchmark
  * main_profiling.py:94-245, which times repeated forwards of one layer): the quadrant sums of
- * W^T -- the five first-level sums, and for two levels the 35 second-level ones -- depend on W
+ * W^T -- the five first-level sums, for two levels the 35 second-level ones, and so on down -- depend on W
  * alone, so they can be formed once and kept in device memory; every forward then forms the
  * input-side sums only.  The reference's LinearStrassen (model/layers.py:246-274) re-forms them
  * on every call.  Results are bit-identical to sthip_linear_forward.
  *
  * sthip_linear_weight_sums_bytes: size of the buffer, or 0 where no sums can be kept (fp32,
- * levels other than 1 or 2, halves -- quarters for two levels -- of in_features not a multiple of
- * 64 or of out_features not a multiple of 128).
+ * levels outside 1..4, in_features / 2^levels not a multiple of 64 or out_features / 2^levels
+ * not a multiple of 128).  1.25 x the bytes of W for one level, 3.4 x for two, 7.3 x for three, 14 x for four:
+ * from three levels on every first-level product keeps the sums of its own weight-side operand.
  * sthip_linear_prepare_weight: forms the sums of W (out x in row-major, 16-byte aligned) into
  * `sums` (256-byte aligned).  Call again whenever W's contents change.
  * sthip_linear_forward_prepared: sthip_linear_forward reading those sums.  A call that does not

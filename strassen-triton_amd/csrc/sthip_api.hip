@@ -355,12 +355,20 @@ static const void* take_bias(const void* C, bool accumulate, bool out_f32) {
 // Quadrant sums of a constant B operand formed ahead of the call (sthip_linear_prepare_weight).
 // The level -- or the two fused levels -- that find their B operand at `target` with the same
 // half extents read these and form the A-side sums only.  Layout: five first-level blocks of
-// kh x nh, then (two levels) 35 second-level blocks of kh/2 x nh/2, as in the workspace.
+// kh x nh, then (two levels) 35 second-level blocks of kh/2 x nh/2, as in the workspace; for
+// three levels and more the five first-level blocks, then one such buffer of levels - 1 for the
+// B operand of each of the seven products M1..M7.
 struct PreparedSums {
     const char* sums = nullptr; size_t bytes = 0; const void* target = nullptr;
     int levels = 0; int64_t kh = 0, nh = 0; bool used = false;
 };
 static thread_local PreparedSums g_prep;
+static size_t prepared_bytes(int levels, int64_t kh, int64_t nh) {
+    const size_t first = 5 * align256(kh * nh * 2);
+    if (levels <= 1) return first;
+    if (levels == 2) return first + 35 * align256((kh / 2) * (nh / 2) * 2);
+    return first + 7 * prepared_bytes(levels - 1, kh / 2, nh / 2);
+}
 static const char* take_prepared(const void* B, int levels, int64_t kh, int64_t nh, size_t need) {
     if (!g_prep.sums || B != g_prep.target || levels != g_prep.levels || kh != g_prep.kh || nh != g_prep.nh ||
         g_prep.bytes < need) return nullptr;
@@ -1502,6 +1510,11 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     char* Mbuf = ws + 5 * (sa_b + sb_b);
     char* child_ws = ws + need;
     const size_t child_bytes = ws_bytes - need;
+    // B-side sums of this level and of the levels below formed ahead of the call: read, never written
+    const char* ready = vec && es == 2 && algo == STHIP_STRASSEN && levels >= 3 && B.rs == 1
+                            ? take_prepared(B.p, levels, kh, nh, prepared_bytes(levels, kh, nh)) : nullptr;
+    const size_t child_prep = ready ? prepared_bytes(levels - 1, kh / 2, nh / 2) : 0;
+    if (ready) SB = const_cast<char*>(ready);
 
     if (vec && dt == STHIP_F32) {
         ComboPair pp;
@@ -1514,7 +1527,7 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     } else if (vec) {
         int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, stream);
         if (rc) return rc;
-        rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, stream);
+        if (!ready) rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, stream);
         if (rc) return rc;
     }
 
@@ -1544,8 +1557,15 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             if (rc) return rc;
             b = {SB, nh, 1};
         }
+        const PreparedSums outer = g_prep;
+        if (ready) {
+            g_prep = PreparedSums{};
+            g_prep.sums = ready + 5 * sb_b + (size_t)q * child_prep; g_prep.bytes = child_prep; g_prep.target = b.p;
+            g_prep.levels = levels - 1; g_prep.kh = kh / 2; g_prep.nh = nh / 2;
+        }
         int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, mh, nh, kh, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
                           false, child_ws, child_bytes, stream, true);
+        g_prep = outer;
         if (rc) return rc;
     }
     return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, stream);
@@ -1697,10 +1717,10 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
 }
 
 // Half extents of W^T (in_features x out_features) for which the weight-side sums can be formed
-// ahead of the call: 16-bit operands, one or two levels, halves (quarters) that the grouped paths take.
+// ahead of the call: 16-bit operands, one to four levels, innermost blocks that the grouped paths take.
 static bool weight_sums_shape(int64_t in_features, int64_t out_features, int dtype, int levels) {
     if (dtype != STHIP_BF16 && dtype != STHIP_F16) return false;
-    if (levels != 1 && levels != 2) return false;
+    if (levels < 1 || levels > 4) return false;
     const int64_t q = (int64_t)1 << levels;
     if (in_features <= 0 || out_features <= 0 || in_features % q || out_features % q) return false;
     return fast_shape(dtype, 128, out_features / q, in_features / q);
@@ -1708,17 +1728,43 @@ static bool weight_sums_shape(int64_t in_features, int64_t out_features, int dty
 
 size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features, int dtype, int levels) {
     if (!weight_sums_shape(in_features, out_features, dtype, levels)) return 0;
-    const int64_t kh = in_features / 2, nh = out_features / 2;
-    size_t n = 5 * align256(kh * nh * 2);
-    if (levels == 2) n += 35 * align256((kh / 2) * (nh / 2) * 2);
-    return n;
+    return prepared_bytes(levels, in_features / 2, out_features / 2);
+}
+
+// Sums of the k x n operand B (stored n-major: B.rs == 1) for `levels` levels into `buf`.
+static int prepare_b(int dt, View B, int64_t k, int64_t n, int levels, char* buf, hipStream_t s) {
+    const int64_t kh = k / 2, nh = n / 2;
+    const size_t sb1 = align256(kh * nh * 2);
+    if (levels == 1) return run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, s);
+    if (levels == 2) {
+        const size_t sb2 = align256((kh / 2) * (nh / 2) * 2);
+        Combo2Pair pp;
+        memset(&pp, 0, sizeof(pp));
+        const int64_t nb = fill_combo2(pp.side[0], B, kh / 2, nh / 2, buf, sb1, buf + 5 * sb1, sb2, 1, STHIP_STRASSEN);
+        dim3 grid((unsigned)ceil_div(nb, 256), 1, 1);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, s, pp);
+        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, s, pp);
+        return check_launch("quad_combos2 (weight)");
+    }
+    int rc = run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, s);
+    if (rc) return rc;
+    const size_t child = prepared_bytes(levels - 1, kh / 2, nh / 2);
+    for (int q = 0; q < 7; ++q) {
+        // B operand of product M(q+1) as multiply() forms it: a quadrant in place or a dense sum
+        const Term tb = kBTerms[q];
+        const View b = tb.sign == 0 ? View{B.p + ((int64_t)(tb.a >> 1) * kh * B.rs + (int64_t)(tb.a & 1) * nh * B.cs) * 2, B.rs, B.cs}
+                                    : View{buf + (size_t)kSumB[q] * sb1, 1, kh};
+        rc = prepare_b(dt, b, kh, nh, levels - 1, buf + 5 * sb1 + (size_t)q * child, s);
+        if (rc) return rc;
+    }
+    return STHIP_OK;
 }
 
 int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_features, int dtype, int levels,
                                 void* sums, size_t sums_bytes, void* stream) {
     g_err[0] = 0;
     const size_t need = sthip_linear_weight_sums_bytes(in_features, out_features, dtype, levels);
-    if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d (16-bit, 1 or 2 levels, aligned halves)",
+    if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d (16-bit, 1 to 4 levels, aligned blocks)",
                            (long long)in_features, (long long)out_features, dtype, levels);
     if (!W || !sums) return fail(STHIP_ERR_ARG, "null pointer");
     if (!aligned_to(W, 16)) return fail(STHIP_ERR_ARG, "W must be 16-byte aligned");
@@ -1726,18 +1772,7 @@ int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_
     if (sums_bytes < need) return fail(STHIP_ERR_WORKSPACE, "sums buffer too small: %zu < %zu bytes", sums_bytes, need);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const View B = {reinterpret_cast<const char*>(W), 1, in_features};   // W^T as a view
-    const int64_t kh = in_features / 2, nh = out_features / 2;
-    const size_t sb1 = align256(kh * nh * 2);
-    char* S1 = reinterpret_cast<char*>(sums);
-    if (levels == 1) return run_combos(dtype, B, kh, nh, S1, sb1, 5, kStrB, s);
-    const size_t sb2 = align256((kh / 2) * (nh / 2) * 2);
-    Combo2Pair pp;
-    memset(&pp, 0, sizeof(pp));
-    const int64_t nb = fill_combo2(pp.side[0], B, kh / 2, nh / 2, S1, sb1, S1 + 5 * sb1, sb2, 1, STHIP_STRASSEN);
-    dim3 grid((unsigned)ceil_div(nb, 256), 1, 1);
-    if (dtype == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, s, pp);
-    else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, s, pp);
-    return check_launch("quad_combos2 (weight)");
+    return prepare_b(dtype, B, in_features, out_features, levels, reinterpret_cast<char*>(sums), s);
 }
 
 int sthip_linear_forward_prepared(const void* x, const void* W, const void* sums, size_t sums_bytes, const void* bias, void* y,

@@ -167,7 +167,7 @@ if __name__ == "__main__":
     ap.add_argument("--max-n", type=int, default=16384)
     ap.add_argument("--gpt2", action="store_true", help="GPT-2-small Linear shapes instead of the square grid")
     ap.add_argument("--cache-weight-sums", action="store_true",
-                    help="keep the quadrant sums of the weight between calls (16-bit, depth 1 and 2)")
+                    help="keep the quadrant sums of the weight between calls (16-bit weights)")
     ap.add_argument("--json", default=None, help="write the measured rows to this file as JSON")
     args = ap.parse_args()
     if not torch.cuda.is_available():

@@ -63,7 +63,7 @@ class LinearStrassenRect(nn.Linear):
         assert d_in == self.in_features, "Input dim mismatch"
         x2d = input.reshape(-1, d_in)
         levels = max(1, int(self.depth))
-        sums = self.weight_sums.get(self.weight, levels) if self.cache_weight_sums and levels <= 2 else None
+        sums = self.weight_sums.get(self.weight, levels) if self.cache_weight_sums else None
         y = _RectLinearFn.apply(x2d, self.weight, self.bias, levels, sums)
         return y.view(*batch_dims, self.out_features)
 

@@ -89,7 +89,8 @@ def test_argument_errors_need_no_gpu():
 
 def test_weight_sums_size_and_argument_errors():
     """Sums of a constant weight: five half-size blocks for one level, 35 quarter-size ones more
-    for two; none for fp32, other depths or halves the grouped paths do not take.  Bad buffers are
+    for two; three and four levels keep
+    such a buffer per first-level product; none for fp32, other depths or blocks the grouped paths do not take.  Bad buffers are
     refused before anything is launched."""
     from strassen_hip import _capi
     lib = _capi.load()
@@ -97,7 +98,11 @@ def test_weight_sums_size_and_argument_errors():
     assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 1, 2) == 5 * 512 * 512 * 2 + 35 * 256 * 256 * 2
     assert lib.sthip_linear_weight_sums_bytes(768, 3072, 2, 1) == 5 * 384 * 1536 * 2
     assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 0, 1) == 0      # fp32
-    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 3) == 0      # three levels
+    two_of_half = 5 * 256 * 256 * 2 + 35 * 128 * 128 * 2
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 3) == 5 * 512 * 512 * 2 + 7 * two_of_half
+    assert lib.sthip_linear_weight_sums_bytes(2048, 2048, 2, 4) == 5 * 1024 * 1024 * 2 + 7 * (5 * 512 * 512 * 2 + 7 * two_of_half)
+    assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 4) == 0      # 64-wide blocks of out_features
+    assert lib.sthip_linear_weight_sums_bytes(1 << 16, 1 << 16, 2, 5) == 0   # more than four levels
     assert lib.sthip_linear_weight_sums_bytes(1024, 1024, 2, 0) == 0
     assert lib.sthip_linear_weight_sums_bytes(1000, 1024, 2, 1) == 0      # 500 is no multiple of 64
     assert lib.sthip_linear_weight_sums_bytes(1024, 768, 2, 2) == 0       # 192 is no multiple of 128
