@@ -85,6 +85,26 @@ int sthip_gemm(const void* A, const void* B, void* C,
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K,
                              int in_dtype, int out_dtype, int algo, int levels);
 
+/* sthip_gemm for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same arguments without the
+ * workspace, which is replaced by a buffer of STHIP_STATIC_SCRATCH_BYTES that is part of the
+ * library's device image (every GPU the library runs on holds its own copy until the process
+ * ends).  The call itself allocates and frees nothing.  Same kernels and same bits as
+ * sthip_gemm given sthip_workspace_bytes() of workspace.  A problem whose workspace query
+ * exceeds the buffer is refused with STHIP_ERR_WORKSPACE before anything is launched (the
+ * buffer covers, for example, one level at 4096^3 and two levels at 2048^3 with 16-bit
+ * operands).  The first call on a device looks up the buffer's address on that device; make
+ * it outside graph capture.  All calls on one GPU share that GPU's buffer: calls that overlap
+ * on one GPU (two streams, two host threads) race on it; calls ordered on one stream do not.
+ * Nothing in the buffer has to start at zero: every path writes what it later reads.
+ * No counterpart in the reference (its torch ops allocate freely). */
+#define STHIP_STATIC_SCRATCH_BYTES ((size_t)144 << 20)
+int sthip_gemm_static(const void* A, const void* B, void* C,
+                      int64_t batch, int64_t M, int64_t N, int64_t K,
+                      const int64_t strideA[3], const int64_t strideB[3], const int64_t strideC[3],
+                      int in_dtype, int out_dtype, int algo, int levels, int accumulate,
+                      void* stream);
+
 /* C = A x B for square n x n operands, `levels` Strassen levels; B may be a transposed view
  * (strides in elements).  Replaces strassen_matmul_n_layers(A, B, n_depth, base_dtype)
  * (fixed_strassen.py:59-126, fixed_strassen_fp32_agg.py:58-125) and, for levels = 1,

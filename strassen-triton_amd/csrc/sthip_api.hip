@@ -3,6 +3,7 @@
 // recursion needs.  See include/strassen_hip.h for the contract of every entry point.
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -1582,6 +1583,34 @@ static int check_common(const void* A, const void* B, const void* C, int64_t bat
     return STHIP_OK;
 }
 
+// ------------------------------------------------------------------ static scratch
+// Workspace of sthip_gemm_static: part of the device image, so every GPU that loads the library
+// holds its own copy at its own address.  `scratch` itself is only a host-side handle for the
+// symbol; kernels, and everything else that needs the memory, get the per-device address that
+// hipGetSymbolAddress returns with that device current.
+static __device__ __align__(256) unsigned char scratch[STHIP_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+static int static_scratch(char** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(STHIP_ERR_HIP, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(STHIP_ERR_HIP, "no address for the static scratch buffer on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = reinterpret_cast<char*>(g_scratch_ptr[dev]);
+    return STHIP_OK;
+}
+
 }  // namespace sthip
 
 using namespace sthip;
@@ -1619,6 +1648,24 @@ int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, 
         if (rc) return rc;
     }
     return STHIP_OK;
+}
+
+int sthip_gemm_static(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                      const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
+                      int in_dtype, int out_dtype, int algo, int levels, int accumulate, void* stream) {
+    g_err[0] = 0;
+    int rc = check_common(A, B, C, batch, M, N, K, in_dtype, out_dtype, algo, levels);
+    if (rc) return rc;
+    const size_t need = sthip_workspace_bytes(batch, M, N, K, in_dtype, out_dtype, algo, levels);
+    if (need > STHIP_STATIC_SCRATCH_BYTES)
+        return fail(STHIP_ERR_WORKSPACE, "problem too large for the static scratch buffer: it needs %zu bytes of workspace, "
+                    "the buffer holds %zu; use sthip_gemm with a workspace of that size", need, (size_t)STHIP_STATIC_SCRATCH_BYTES);
+    char* ws = nullptr;
+    if (need > 0) {
+        rc = static_scratch(&ws);
+        if (rc) return rc;
+    }
+    return sthip_gemm(A, B, C, batch, M, N, K, sA, sB, sC, in_dtype, out_dtype, algo, levels, accumulate, ws, need, stream);
 }
 
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {

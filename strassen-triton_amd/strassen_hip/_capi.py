@@ -17,6 +17,8 @@ _p64 = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "sthip_gemm": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _p64, _p64, _p64,
                           _int, _int, _int, _int, _int, _vp, _sz, _vp]),
+    "sthip_gemm_static": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _p64, _p64, _p64,
+                                 _int, _int, _int, _int, _int, _vp]),
     "sthip_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _int, _int, _int]),
     "sthip_strassen_matmul_n_layers": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                               _int, _int, _vp, _sz, _vp]),

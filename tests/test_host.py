@@ -44,6 +44,12 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_gemm(one, one, one, 1, 0, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None, 0, None) == 0   # empty M
     assert lib.sthip_linear_strassen_forward(one, one, None, one, 9, 8, 0, 1, None, 0, None) == -1
     assert b"cannot be padded" in lib.sthip_last_error()
+    # the entry point that brings its own scratch refuses a problem whose workspace exceeds that buffer
+    wide = (ctypes.c_int64 * 3)(0, 8192, 1)
+    assert lib.sthip_gemm_static(one, one, one, 1, 8192, 8192, 8192, wide, wide, wide, 2, 2, 1, 1, 0, None) == -4
+    assert b"static scratch" in lib.sthip_last_error()
+    assert lib.sthip_gemm_static(one, one, one, 1, -1, 4, 4, s3, s3, s3, 0, 0, 1, 1, 0, None) == -1
+    assert lib.sthip_workspace_bytes(1, 4096, 4096, 4096, 2, 2, 1, 1) <= 144 << 20 < lib.sthip_workspace_bytes(1, 8192, 8192, 8192, 2, 2, 1, 1)
     # two or more levels need the workspace the query asks for: refused before anything is launched
     big = (ctypes.c_int64 * 3)(0, 1024, 1)
     for dt in (0, 2):
