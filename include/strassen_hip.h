@@ -4,6 +4,7 @@
  * knows about torch.  All work is enqueued on the HIP stream passed in (NULL = the default
  * stream) and nothing synchronises.  The library never allocates or frees device memory:
  * the multi-level paths take a caller-provided workspace (sthip_workspace_bytes).
+ * Test and profiling hooks live in strassen_hip_debug.h, not here.
  *
  * Return value: 0 on success, a negative sthip_status otherwise; sthip_last_error() then
  * describes the failure (thread local).
@@ -174,21 +175,6 @@ const char* sthip_last_error(void);
 
 /* STHIP_VERSION the library was built with. */
 int sthip_version(void);
-
-/* Diagnostic: runs the 16-bit transposing LDS read on a 64 x 4 grid of 16-bit values
- * (value = 4 * lane + element) and writes what each lane received to out[64 * 4] (uint16,
- * device memory).  Used by the tests to pin the lane mapping the kernels rely on.  No
- * counterpart in the reference. */
-int sthip_debug_transpose_read(void* out, void* stream);
-
-/* Profiling aid: selects which stages of the pipelined one-level path later calls run
- * (bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM, bit 2 = recombination pass of the
- * grouped paths; bit 3 lets two-level calls run as one 49-product launch instead of the host
- * recursion, bit 4 lets that form recombine 49 -> C in one pass instead of two, bit 5 lets it
- * form the sums of both levels in one pass instead of two; default 63) and returns the previous mask.  With mask 2 the GEMM re-uses the
- * sums a previous call left in the same workspace, so the dominant kernel can be timed alone.
- * Process-wide; not for production calls.  No counterpart in the reference. */
-int sthip_debug_set_stages(int mask);
 
 #ifdef __cplusplus
 }

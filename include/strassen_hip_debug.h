@@ -1,0 +1,35 @@
+/* strassen_hip_debug.h -- test and profiling hooks of libstrassen_hip.so.  Not part of the
+ * drop-in boundary (strassen_hip.h); none of them has a counterpart in the reference.  The two
+ * switches are process-wide: every public entry point reads them once when it is called, so a
+ * change never affects a call that is already running, but it does affect other threads' later
+ * calls.  Not for production code. */
+#ifndef STRASSEN_HIP_DEBUG_H
+#define STRASSEN_HIP_DEBUG_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Runs the 16-bit transposing LDS read on a 64 x 4 grid of 16-bit values (value = 4 * lane +
+ * element) and writes what each lane received to out[64 * 4] (uint16, device memory).  Used by
+ * the tests to pin the lane mapping the kernels rely on. */
+int sthip_debug_transpose_read(void* out, void* stream);
+
+/* Selects which stages of the pipelined paths later calls run (bit 0 = quadrant-sum pre-pass,
+ * bit 1 = grouped GEMM, bit 2 = recombination pass; bit 3 lets two-level calls run as one
+ * 49-product launch instead of the host recursion; default 15) and returns the previous mask.
+ * With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so the
+ * dominant kernel can be timed alone. */
+int sthip_debug_set_stages(int mask);
+
+/* Overrides the tile table for later calls where the shape allows the forced tile: "128x128",
+ * "256x128" (kernels that recombine in registers), "128x128g", "256x256" (grouped products);
+ * NULL or anything else = automatic.  Returns the previous setting as a code (0 = automatic).
+ * The environment variable STHIP_FORCE_TILE gives the initial setting; it is read once, by the
+ * first call into the library. */
+int sthip_debug_force_tile(const char* tile);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STRASSEN_HIP_DEBUG_H */

@@ -54,7 +54,8 @@ def _digest(extra):
         if os.path.isfile(path):
             h.update(name.encode())
             h.update(open(path, "rb").read())
-    h.update(open(os.path.join(HERE, "..", "include", "strassen_hip.h"), "rb").read())
+    for hdr in ("strassen_hip.h", "strassen_hip_debug.h"):
+        h.update(open(os.path.join(HERE, "..", "include", hdr), "rb").read())
     h.update(" ".join(FLAGS + extra).encode())
     return h.hexdigest()
 

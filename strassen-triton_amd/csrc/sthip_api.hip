@@ -3,6 +3,7 @@
 // recursion needs.  See include/strassen_hip.h for the contract of every entry point.
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
@@ -10,16 +11,21 @@
 #include <string.h>
 
 #include "../../include/strassen_hip.h"
+#include "../../include/strassen_hip_debug.h"
 #include "sthip_launch.hpp"
 
 namespace sthip {
 
 static thread_local char g_err[512] = "";
-// Which stages of the pipelined path run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
-// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch, bit 4 = that
-// form recombines 49 -> C in one pass instead of two, bit 5 = and forms the sums of both levels in
-// one pass instead of two.  Only the profiling hook sthip_debug_set_stages changes it.
-static int g_stages = 63;
+// Process-wide debug switches (include/strassen_hip_debug.h).  Every public entry point reads them
+// once, into its Call; nothing below an entry point looks at them again.
+// Stages of the pipelined path that run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
+// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch.
+constexpr int kAllStages = 15;
+static std::atomic<int> g_debug_stages{kAllStages};
+// Forced tile: 0 = the tile table decides, 2 = 128 x 128, 3 = 256 x 128, 4 = 256 x 256, 5 = 128 x 128 with
+// the seven products as separate outputs; -1 = not set yet (the first call reads STHIP_FORCE_TILE).
+static std::atomic<int> g_debug_tile{-1};
 
 static int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -71,16 +77,25 @@ static const LaunchTable3* table4_for(int dt) {
     return dt == STHIP_F32 ? &kLaunch4_0 : dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
 }
 
-// STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 overrides the tile table where the shape allows
-// the forced tile (tuning and test aid); unset or anything else = automatic.
-static int forced_tile() {
-    const char* e = getenv("STHIP_FORCE_TILE");
+// STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 in the environment of the process overrides the
+// tile table where the shape allows the forced tile (tuning aid); it is read once, by the first call.
+// sthip_debug_force_tile changes the setting later.
+static int tile_code(const char* e) {
     if (!e) return 0;
     if (!strcmp(e, "128x128")) return 2;
     if (!strcmp(e, "256x128")) return 3;
     if (!strcmp(e, "256x256")) return 4;
     if (!strcmp(e, "128x128g")) return 5;   // 128 x 128 tiles, seven products as separate outputs
     return 0;
+}
+static int forced_tile_setting() {
+    int t = g_debug_tile.load(std::memory_order_relaxed);
+    if (t < 0) {
+        t = tile_code(getenv("STHIP_FORCE_TILE"));
+        int expected = -1;
+        if (!g_debug_tile.compare_exchange_strong(expected, t)) t = expected;
+    }
+    return t;
 }
 
 static bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -174,12 +189,6 @@ __global__ void __launch_bounds__(256) quad_combos_pair_kernel(const ComboPair p
 
 __global__ void __launch_bounds__(256) quad_combos_pair_f32_kernel(const ComboPair pp) { quad_combos_f32_body(pp.side[blockIdx.z]); }
 
-// The fourteen operands of the seven products of a level (second-level sums) in one launch.
-struct ComboMany { ComboParams side[14]; };
-template <class T>
-__global__ void __launch_bounds__(256) quad_combos_many_kernel(const ComboMany pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
-__global__ void __launch_bounds__(256) quad_combos_many_f32_kernel(const ComboMany pp) { quad_combos_f32_body(pp.side[blockIdx.z]); }
-
 // Eight 16-bit elements of a 16-byte chunk as floats.
 template <class T>
 __device__ __forceinline__ void unpack8(const u32x4 v, float* x) {
@@ -230,12 +239,12 @@ __device__ __forceinline__ typename ElemVec<T>::type pack_elems(const float* x) 
 }
 
 // The sums of BOTH levels of a two-level product for one operand in one pass: the sixteen quarter
-// blocks are read once; every first-level operand (a quadrant, or a sum of two rounded to the
-// operand type as the two-pass form stores it) is formed in registers, the quarters of the
+// blocks are read once; every first-level operand (a quadrant, or a sum of two rounded once to
+// the operand type, fixed_strassen_fp32_agg.py:87-96) is formed in registers, the quarters of the
 // first-level sums that the second level multiplies directly are stored, and so are the
-// second-level sums of all seven first-level operands.  Same additions in the same order as
-// quad_combos_body, so the outputs are bit-identical to the two passes -- without writing the
-// other half of the first-level sums and without re-reading any of them.
+// second-level sums of all seven first-level operands (fp32 sums of the rounded first-level
+// values, rounded once).  The other half of the first-level sums is never written and none is
+// re-read.
 struct Combo2Params {
     const void* x[16];        // quarter blocks of the operand, logical (R, C) -> x[4 R + C]
     void* s1[5];              // first-level sums: dense half-size blocks in the operand's storage orientation
@@ -343,15 +352,9 @@ struct Recombine16Params {
                                   // result and the sum rounded again, as a separate add would (model/layers.py:271-272)
 };
 
-// Bias of the Linear forward in flight on this thread: the recombination pass that writes `target`
-// adds it, so that no separate pass over the output is needed.
+// Bias of a Linear forward: the recombination pass that writes `target` adds it, so that no
+// separate pass over the output is needed.
 struct BiasEpilogue { const void* bias = nullptr; const void* target = nullptr; bool applied = false; };
-static thread_local BiasEpilogue g_bias;
-static const void* take_bias(const void* C, bool accumulate, bool out_f32) {
-    if (!g_bias.bias || C != g_bias.target || accumulate || out_f32) return nullptr;
-    g_bias.applied = true;
-    return g_bias.bias;
-}
 
 // Quadrant sums of a constant B operand formed ahead of the call (sthip_linear_prepare_weight).
 // The level -- or the two fused levels -- that find their B operand at `target` with the same
@@ -361,20 +364,35 @@ static const void* take_bias(const void* C, bool accumulate, bool out_f32) {
 // B operand of each of the seven products M1..M7.
 struct PreparedSums {
     const char* sums = nullptr; size_t bytes = 0; const void* target = nullptr;
-    int levels = 0; int64_t kh = 0, nh = 0; bool used = false;
+    int levels = 0; int64_t kh = 0, nh = 0;
 };
-static thread_local PreparedSums g_prep;
+
+// What a public entry point decides once and everything below it shares: the stream, the debug
+// switches as they stood at entry, the bias a Linear forward wants added by its last pass, and
+// the weight-side sums formed ahead of the call.
+struct Call {
+    hipStream_t stream = nullptr;
+    int stages = kAllStages;
+    int force_tile = 0;
+    BiasEpilogue bias;
+    PreparedSums prep;
+};
+
+static const void* take_bias(Call& cx, const void* C, bool accumulate, bool out_f32) {
+    if (!cx.bias.bias || C != cx.bias.target || accumulate || out_f32) return nullptr;
+    cx.bias.applied = true;
+    return cx.bias.bias;
+}
 static size_t prepared_bytes(int levels, int64_t kh, int64_t nh) {
     const size_t first = 5 * align256(kh * nh * 2);
     if (levels <= 1) return first;
     if (levels == 2) return first + 35 * align256((kh / 2) * (nh / 2) * 2);
     return first + 7 * prepared_bytes(levels - 1, kh / 2, nh / 2);
 }
-static const char* take_prepared(const void* B, int levels, int64_t kh, int64_t nh, size_t need) {
-    if (!g_prep.sums || B != g_prep.target || levels != g_prep.levels || kh != g_prep.kh || nh != g_prep.nh ||
-        g_prep.bytes < need) return nullptr;
-    g_prep.used = true;
-    return g_prep.sums;
+static const char* take_prepared(const Call& cx, const void* B, int levels, int64_t kh, int64_t nh, size_t need) {
+    const PreparedSums& ps = cx.prep;
+    if (!ps.sums || B != ps.target || levels != ps.levels || kh != ps.kh || nh != ps.nh || ps.bytes < need) return nullptr;
+    return ps.sums;
 }
 
 
@@ -451,12 +469,11 @@ __global__ void __launch_bounds__(256) recombine16_kernel(const Recombine16Param
 
 // Both recombinations of a two-level product in one pass: from the 49 quarter-size 16-bit products
 // (first-level product p, second-level product k at prod + (7 p + k) * p_ps) straight to C.  The
-// second-level result of every first-level product is rounded to the operand type in registers,
-// exactly where the two-pass form stores it, and the first level adds in the same order as
-// recombine16_kernel (p visited in the order 4 6 5 2 0 3 1 gives each quadrant its terms in that
-// order), so the result is bit-identical to the two passes -- without writing and re-reading the
-// seven half-size products.  One thread per 16-byte chunk of a quarter-size row; Mh, Nh are the
-// quarter sizes here.
+// second-level result of every first-level product stays in fp32 registers (the reference's inner
+// call returns fp32 as well, fixed_strassen_fp32_agg.py:99-106) and the first level adds in the
+// same order as recombine16_kernel (p visited in the order 4 6 5 2 0 3 1 gives each quadrant its
+// terms in that order); the seven half-size products are never written.  One thread per 8-byte
+// chunk of a quarter-size row; Mh, Nh are the quarter sizes here.
 
 template <class T, int ALGO2>
 __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Params p) {
@@ -468,7 +485,7 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
     const int i = (int)(idx / nq), j = (int)(idx % nq) * E;
     const char* src = reinterpret_cast<const char*>(p.prod) + ((int64_t)i * p.Nh + j) * ES;
     float acc[4][4][E];   // [quadrant of C][quarter block within it][element]
-    // second level of first-level product pp -> m[quarter block][element], rounded to T
+    // second level of first-level product pp -> m[quarter block][element], fp32
     auto second = [&](int pp, float (&m)[4][E]) {
         float x[7][E];
 #pragma unroll
@@ -488,8 +505,6 @@ __global__ void __launch_bounds__(256) recombine16x2_kernel(const Recombine16Par
                 m[2][e] = u3 + x[6][e];
                 m[3][e] = u3 + x[4][e];
             }
-#pragma unroll
-            for (int b = 0; b < 4; ++b) m[b][e] = round16<T>(m[b][e]);
         }
     };
     float m[4][E];
@@ -593,7 +608,7 @@ static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
 // Returns 1 if the problem does not qualify (the caller then takes the fused kernel).
 static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch, int64_t a_bs, int64_t b_bs,
                             int64_t c_bs, int64_t Mh, int64_t Nh, int64_t Kh, int dt, bool out_f32, int algo,
-                            bool accumulate, bool a_kc, bool b_kc, char* ws, size_t ws_bytes, hipStream_t stream) {
+                            bool accumulate, bool a_kc, bool b_kc, char* ws, size_t ws_bytes, Call& cx) {
     const bool split = algo != STHIP_CLASSIC;
     if (split && (!ws || !aligned_to(ws, 256) || ws_bytes < prepass_bytes(batch, Mh, Nh, Kh))) return 1;
     const int64_t a_ld = a_kc ? A.rs : A.cs, b_ld = b_kc ? B.cs : B.rs;
@@ -615,13 +630,13 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2);
         char* SA = ws;                                // [5][batch] blocks of Mh x Kh (storage order of A)
         char* SB = ws + (size_t)batch * 5 * sa_b;
-        const char* ready = algo == STHIP_STRASSEN && batch == 1 && b_kc ? take_prepared(B.p, 1, Kh, Nh, 5 * sb_b) : nullptr;
+        const char* ready = algo == STHIP_STRASSEN && batch == 1 && b_kc ? take_prepared(cx, B.p, 1, Kh, Nh, 5 * sb_b) : nullptr;
         if (ready) SB = const_cast<char*>(ready);     // B-side sums formed ahead of the call: read, never written
         // region after the sums: parked fp32 tiles (256 x 128 kernel) or the seven 16-bit products (grouped paths)
         p.park = reinterpret_cast<float*>(ws + (size_t)batch * 5 * (sa_b + sb_b));
         const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
         const int nout = algo == STHIP_STRASSEN ? 5 : 4;
-        if (g_stages & 1) {
+        if (cx.stages & 1) {
             ComboPair pp;
             memset(&pp, 0, sizeof(pp));
             int64_t most = 0;
@@ -645,8 +660,8 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
                 most = std::max(most, r_ext * (c_ext / 8));
             }
             dim3 grid((unsigned)ceil_div(most, 256), (unsigned)batch, (unsigned)sides);
-            if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
-            else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
+            if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, cx.stream, pp);
+            else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, cx.stream, pp);
             int rc = check_launch("quad_combos");
             if (rc) return rc;
         }
@@ -687,7 +702,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
     hipError_t e = hipSuccess;
     const LaunchTable3* t3 = table3_for(dt, algo);
     const LaunchTable3* t4 = table4_for(dt);
-    const int force = forced_tile();
+    const int force = cx.force_tile;
     const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
     // products as matrices + recombination pass: 16-bit products for a result in the operand type,
     // fp32 products (twice the room) for an fp32 result
@@ -718,31 +733,31 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
         rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0; rp.p_ps = Mh * Nh; rp.out_f32 = out_f32 ? 1 : 0;
-        if (batch == 1 && (g_stages & 4)) rp.bias = take_bias(C, accumulate, out_f32);
-        if (g_stages & 2) {
+        if (batch == 1 && (cx.stages & 4)) rp.bias = take_bias(cx, C, accumulate, out_f32);
+        if (cx.stages & 2) {
             p.C = p.park; p.c_rs = Nh; p.c_ps = Mh * Nh; p.c_bs = 7 * Mh * Nh;
             p.out_f32 = out_f32 ? 1 : 0; p.accumulate = 0; p.nprod = 7;
             if (pick == 4) {
                 p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
                 p.group_m = 4;
                 p.c_wide = wide_rows(p.C, p.c_rs, p.c_ps, p.c_bs);
-                e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+                e = t4->fn[b_kc ? 1 : 0](p, (int)batch, cx.stream);
             } else {
                 const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
                 if (!t) return 1;
-                e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+                e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, cx.stream);
             }
             if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
         }
-        if ((g_stages & 4) && out_f32) {
+        if ((cx.stages & 4) && out_f32) {
             dim3 grid((unsigned)ceil_div(Mh * (Nh / 4), 256), (unsigned)batch);
-            if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, stream, rp);
-            else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, stream, rp);
+            if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, cx.stream, rp);
+            else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, cx.stream, rp);
             return check_launch("recombine32");
         }
-        if (g_stages & 4) {
+        if (cx.stages & 4) {
             dim3 grid((unsigned)ceil_div(Mh * (Nh / 8), 256), (unsigned)batch);
-#define GO(T, A) hipLaunchKernelGGL((recombine16_kernel<T, A>), grid, dim3(256), 0, stream, rp)
+#define GO(T, A) hipLaunchKernelGGL((recombine16_kernel<T, A>), grid, dim3(256), 0, cx.stream, rp)
             if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
             else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
 #undef GO
@@ -750,20 +765,20 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         }
         return STHIP_OK;
     }
-    if (!(g_stages & 2)) return STHIP_OK;
+    if (!(cx.stages & 2)) return STHIP_OK;
     if (pick == 4) {
         p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
         p.group_m = 4; p.nprod = 1;
         p.c_wide = wide_rows(p.C, p.c_rs, 0, p.c_bs);
-        e = t4->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+        e = t4->fn[b_kc ? 1 : 0](p, (int)batch, cx.stream);
     } else if (pick == 3) {
         p.tiles_m = (int)(Mh / kBM3);
         p.group_m = 4;
-        e = t3->fn[b_kc ? 1 : 0](p, (int)batch, stream);
+        e = t3->fn[b_kc ? 1 : 0](p, (int)batch, cx.stream);
     } else {
         const LaunchTable2* t = table2_for(dt, algo);
         if (!t) return 1;
-        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, stream);
+        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](p, (int)batch, cx.stream);
     }
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
     return STHIP_OK;
@@ -775,15 +790,15 @@ static size_t f32_batched_bytes(int64_t Mh, int64_t Nh, int64_t Kh) {
     return 7 * (align256(Mh * Kh * 4) + align256(Kh * Nh * 4) + align256(Mh * Nh * 4));
 }
 static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 bool accumulate, char* ws, hipStream_t stream);
+                                 bool accumulate, char* ws, Call& cx);
 static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 int algo, bool accumulate, char* ws, hipStream_t stream);
+                                 int algo, bool accumulate, char* ws, Call& cx);
 
 static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                         int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
                         int64_t M, int64_t N, int64_t K, int64_t Mh, int64_t Nh, int64_t Kh,
                         int dt, bool out_f32, int algo, bool accumulate, char* ws, size_t ws_bytes,
-                        hipStream_t stream) {
+                        Call& cx) {
     if (M == 0 || N == 0 || batch == 0) return STHIP_OK;
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || batch > 65535)
         return fail(STHIP_ERR_SHAPE, "size out of range (M=%lld N=%lld K=%lld batch=%lld)",
@@ -830,14 +845,14 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
 
     if (fast && fast_shape(dt, Mh, Nh, Kh) && a_long % 8 == 0 && b_long % 8 == 0) {
         int rc = launch_pipelined(A, B, C, c_rs, batch, a_bs, b_bs, c_bs, Mh, Nh, Kh, dt, out_f32, algo, accumulate,
-                                  a_kc, b_kc, ws, ws_bytes, stream);
+                                  a_kc, b_kc, ws, ws_bytes, cx);
         if (rc <= 0) return rc;
     }
     // fp32 on the 256 x 256 pipelined kernel (A contiguous along k, enough tiles to fill the chip):
     // a classical product directly; one Strassen level as sums, ONE grouped launch of the seven
     // products and the recombination pass.  Measured at 8192^3: the classical product runs at
     // 142 TFLOP/s against 85 on the fused kernel.
-    if (fast && dt == STHIP_F32 && a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && Kh % 32 == 0 && forced_tile() != 2) {
+    if (fast && dt == STHIP_F32 && a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && Kh % 32 == 0 && cx.force_tile != 2) {
         const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch;
         if (!split && tiles4 >= 224) {
             Gemm2Params g;
@@ -847,23 +862,23 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             g.Mh = (int)Mh; g.Nh = (int)Nh; g.Kh = (int)Kh;
             g.tiles_m = (int)(Mh / kBM4); g.tiles_n = (int)(Nh / kBN4);
             g.out_f32 = 1; g.accumulate = accumulate ? 1 : 0; g.group_m = 4; g.nprod = 1;
-            hipError_t e = table4_for(dt)->fn[b_kc ? 1 : 0](g, (int)batch, stream);
+            hipError_t e = table4_for(dt)->fn[b_kc ? 1 : 0](g, (int)batch, cx.stream);
             if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
             return STHIP_OK;
         }
         if (split && batch == 1 && 7 * tiles4 >= 224 && ws && aligned_to(ws, 256) &&
             ws_bytes >= f32_batched_bytes(Mh, Nh, Kh))
-            return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, algo, accumulate, ws, stream);
+            return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, algo, accumulate, ws, cx);
     }
     // fp32, one Strassen level: run the seven products side by side as a batch (see
     // one_level_f32_batched).  Measured against the fused kernel: 5 x faster at 1024^3 (one product
     // has 16 tiles for 256 CUs), 3 x at 2048^3, equal at 4096^3, 10 % faster at 8192^3.
     if (fast && dt == STHIP_F32 && algo == STHIP_STRASSEN && batch == 1 && ws && aligned_to(ws, 256) &&
-        ws_bytes >= f32_batched_bytes(Mh, Nh, Kh) && forced_tile() != 2)
-        return one_level_f32_batched(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, stream);
+        ws_bytes >= f32_batched_bytes(Mh, Nh, Kh) && cx.force_tile != 2)
+        return one_level_f32_batched(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, cx);
     const LaunchTable* t = table_for(dt, algo);
     if (!t) return fail(STHIP_ERR_ARG, "bad dtype/algo (%d, %d)", dt, algo);
-    hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0][fast ? 0 : 1](p, (int)batch, stream);
+    hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0][fast ? 0 : 1](p, (int)batch, cx.stream);
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
     return STHIP_OK;
 }
@@ -986,13 +1001,13 @@ static int64_t fill_combo(ComboParams& cp, View X, int64_t r_blk, int64_t c_blk,
 }
 
 static int run_combos(int dt, View X, int64_t r_blk, int64_t c_blk, char* out, size_t out_stride, int nout,
-                      const signed char (*coef)[4], hipStream_t stream) {
+                      const signed char (*coef)[4], Call& cx) {
     ComboParams cp;
     const int64_t n = fill_combo(cp, X, r_blk, c_blk, out, out_stride, nout, coef);
     if (n == 0) return STHIP_OK;
     dim3 grid((unsigned)ceil_div(n, 256), 1);
-    if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, stream, cp);
-    else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, stream, cp);
+    if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_kernel<bf16_t>, grid, dim3(256), 0, cx.stream, cp);
+    else hipLaunchKernelGGL(quad_combos_kernel<f16_t>, grid, dim3(256), 0, cx.stream, cp);
     return check_launch("quad_combos");
 }
 
@@ -1023,20 +1038,6 @@ static void level_operands(int algo, View A, View B, int64_t mh, int64_t nh, int
         xa[5] = sumA(3); xb[5] = rawB(3);   // P3 = S4 B22
         xa[6] = rawA(3); xb[6] = sumB(3);   // -P4 = A22 (-T4)
     }
-}
-
-static int launch_recombine16(int dt, int algo, const void* prod, int64_t p_ps, char* C, int64_t c_rs, int64_t c_bs,
-                              int64_t batch, int64_t Mh, int64_t Nh, bool accumulate, bool out_f32, hipStream_t stream) {
-    Recombine16Params rp;
-    rp.out_f32 = out_f32 ? 1 : 0;
-    rp.prod = prod; rp.p_ps = p_ps; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
-    rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
-    dim3 grid((unsigned)ceil_div(Mh * (Nh / 8), 256), (unsigned)batch);
-#define GO(T, A) hipLaunchKernelGGL((recombine16_kernel<T, A>), grid, dim3(256), 0, stream, rp)
-    if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
-    else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
-#undef GO
-    return check_launch("recombine16");
 }
 
 // One operand of quad_combos2_kernel.  X is the whole operand, (rq, cq) the quarter-block size in
@@ -1083,15 +1084,17 @@ static int64_t fill_combo2(Combo2Params& cp, View X, int64_t rq, int64_t cq, cha
 // Two levels as three launches: the sums of both levels in one pass over the operands, ONE
 // grouped GEMM of the 49 quarter-size products (the schedule the reference's two-layer Triton
 // kernel runs per tile, strassen.py:373-611, here on whole matrices), both recombinations in one
-// pass.  Every level returns its result in the operand type, as the reference's recursion does
-// (fixed_strassen_fp32_agg.py:47-50): the passes round in registers where the five-launch form
-// (sums 1, sums 2, GEMM, 49 -> 7, 7 -> C; stage-mask bits 4 and 5 off) rounds on its way through
-// memory, and give the same bits.  The first level is always Strassen.
+// pass.  Cast schedule: first-level sums rounded once to the operand type, as the reference rounds
+// them (fixed_strassen_fp32_agg.py:87-96); second-level sums formed in fp32 from those and rounded
+// once (the reference multiplies them unrounded, in fp32, :99-113 -- here the inner products run
+// on the 16-bit matrix cores); the 49 products rounded to the operand type as every product of this
+// library is; both recombinations in fp32 with no rounding between them, as the reference's inner
+// call returns fp32 (:99-106); one final rounding.  The first level is always Strassen.
 // Needs: 16-bit operands, whole aligned problem, C in the operand type with 16-byte aligned rows.
 static size_t two_level_bytes(int64_t mh, int64_t nh, int64_t kh) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     return 5 * (align256(mh * kh * 2) + align256(kh * nh * 2)) + 35 * (align256(mq * kq * 2) + align256(kq * nq * 2)) +
-           49 * align256(mq * nq * 2) + 7 * align256(mh * nh * 2);
+           49 * align256(mq * nq * 2);
 }
 
 static bool two_level_shape(int dt, int64_t mh, int64_t nh, int64_t kh) {
@@ -1099,64 +1102,35 @@ static bool two_level_shape(int dt, int64_t mh, int64_t nh, int64_t kh) {
 }
 
 static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int64_t nh, int64_t kh,
-                          int dt, int algo, bool accumulate, bool out_f32, char* ws, hipStream_t stream) {
+                          int dt, int algo, bool accumulate, bool out_f32, char* ws, Call& cx) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     const size_t sa1 = align256(mh * kh * 2), sb1 = align256(kh * nh * 2);
     const size_t sa2 = align256(mq * kq * 2), sb2 = align256(kq * nq * 2);
-    const size_t pb = align256(mq * nq * 2), mb = align256(mh * nh * 2);
+    const size_t pb = align256(mq * nq * 2);
     char* SA1 = ws;
     char* SB1 = SA1 + 5 * sa1;
     char* SA2 = SB1 + 5 * sb1;
     char* SB2 = SA2 + 35 * sa2;
     char* P = SB2 + 35 * sb2;
-    char* Mp = P + 49 * pb;
     const bool a_kc = A.cs == 1, b_kc = B.rs == 1;
     const int nout2 = algo == STHIP_STRASSEN ? 5 : 4;
     // B-side sums of both levels formed ahead of the call: read, never written
-    const char* ready = algo == STHIP_STRASSEN && b_kc && (g_stages & 32) ? take_prepared(B.p, 2, kh, nh, 5 * sb1 + 35 * sb2) : nullptr;
+    const char* ready = algo == STHIP_STRASSEN && b_kc ? take_prepared(cx, B.p, 2, kh, nh, 5 * sb1 + 35 * sb2) : nullptr;
     if (ready) { SB1 = const_cast<char*>(ready); SB2 = SB1 + 5 * sb1; }
 
-    // sums of both levels in one pass (bit 5 of the stage mask off: as two passes)
-    if ((g_stages & 32) && (g_stages & 1)) {
+    // sums of both levels in one pass
+    if (cx.stages & 1) {
         Combo2Pair pp;
         const int64_t na = fill_combo2(pp.side[0], A, mq, kq, SA1, sa1, SA2, sa2, 0, algo);
         const int64_t nb = ready ? 0 : fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, algo);
         dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, ready ? 1 : 2);
-        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
-        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, cx.stream, pp);
+        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, cx.stream, pp);
         int rc = check_launch("quad_combos2");
-        if (rc) return rc;
-    }
-    // first-level sums (Strassen)
-    if (!(g_stages & 32) && (g_stages & 1)) {
-        ComboPair pp;
-        const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA);
-        const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB);
-        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_pair_kernel<bf16_t>, grid, dim3(256), 0, stream, pp);
-        else hipLaunchKernelGGL(quad_combos_pair_kernel<f16_t>, grid, dim3(256), 0, stream, pp);
-        int rc = check_launch("quad_combos (level 1)");
         if (rc) return rc;
     }
     View xa1[7], xb1[7];
     level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1);
-
-    // second-level sums of all fourteen operands
-    if (!(g_stages & 32) && (g_stages & 1)) {
-        ComboMany pm;
-        int64_t most = 0;
-        for (int p = 0; p < 7; ++p) {
-            most = std::max(most, fill_combo(pm.side[2 * p], xa1[p], mq, kq, SA2 + (size_t)p * 5 * sa2, sa2, nout2,
-                                             algo == STHIP_STRASSEN ? kStrA : kWinA));
-            most = std::max(most, fill_combo(pm.side[2 * p + 1], xb1[p], kq, nq, SB2 + (size_t)p * 5 * sb2, sb2, nout2,
-                                             algo == STHIP_STRASSEN ? kStrB : kWinB));
-        }
-        dim3 grid((unsigned)ceil_div(most, 256), 1, 14);
-        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos_many_kernel<bf16_t>, grid, dim3(256), 0, stream, pm);
-        else hipLaunchKernelGGL(quad_combos_many_kernel<f16_t>, grid, dim3(256), 0, stream, pm);
-        int rc = check_launch("quad_combos (level 2)");
-        if (rc) return rc;
-    }
 
     // the 49 products, product-major: first-level product p, second-level product j -> P[7 p + j]
     Gemm2Params g;
@@ -1171,36 +1145,30 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     g.Mh = (int)mq; g.Nh = (int)nq; g.Kh = (int)kq;
     g.out_f32 = 0; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
     const LaunchTable3* t4 = table4_for(dt);
-    const bool big = a_kc && t4 && mq % kBM4 == 0 && nq % kBN4 == 0 && kq >= 1024 && forced_tile() != 5 && forced_tile() != 2;
+    const bool big = a_kc && t4 && mq % kBM4 == 0 && nq % kBN4 == 0 && kq >= 1024 && cx.force_tile != 5 && cx.force_tile != 2;
     hipError_t e = hipSuccess;
-    if (!(g_stages & 2)) {
+    if (!(cx.stages & 2)) {
     } else if (big) {
         g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
         g.c_wide = wide_rows(g.C, g.c_rs, g.c_ps, 0);
-        e = t4->fn[b_kc ? 1 : 0](g, 1, stream);
+        e = t4->fn[b_kc ? 1 : 0](g, 1, cx.stream);
     } else {
         const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
         if (!t) return fail(STHIP_ERR_DTYPE, "no 16-bit kernel for dtype %d", dt);
         g.tiles_m = (int)(mq / 128); g.tiles_n = (int)(nq / 128);
         g.group_m = 8;
-        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](g, 1, stream);
+        e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0](g, 1, cx.stream);
     }
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
 
-    // 49 -> C: both recombinations in one pass (bit 4 of the stage mask off: as two passes, 49 -> 7
-    // with one batch entry per first-level product, then 7 -> C)
-    if (!(g_stages & 4)) return STHIP_OK;
-    if (!(g_stages & 16)) {
-        int rc = launch_recombine16(dt, algo, P, (int64_t)(pb / 2), Mp, nh, (int64_t)(mb / 2), 7, mq, nq, false, false, stream);
-        if (rc) return rc;
-        return launch_recombine16(dt, STHIP_STRASSEN, Mp, (int64_t)(mb / 2), C, c_rs, 0, 1, mh, nh, accumulate, out_f32, stream);
-    }
+    // 49 -> C: both recombinations in one pass
+    if (!(cx.stages & 4)) return STHIP_OK;
     Recombine16Params rp;
     rp.prod = P; rp.p_ps = (int64_t)(pb / 2); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
     rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = out_f32 ? 1 : 0;
-    rp.bias = take_bias(C, accumulate, out_f32);
+    rp.bias = take_bias(cx, C, accumulate, out_f32);
     dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
-#define GO(T, A) hipLaunchKernelGGL((recombine16x2_kernel<T, A>), grid, dim3(256), 0, stream, rp)
+#define GO(T, A) hipLaunchKernelGGL((recombine16x2_kernel<T, A>), grid, dim3(256), 0, cx.stream, rp)
     if (dt == STHIP_BF16) { if (algo == STHIP_STRASSEN) GO(bf16_t, STHIP_STRASSEN); else GO(bf16_t, STHIP_WINOGRAD); }
     else { if (algo == STHIP_STRASSEN) GO(f16_t, STHIP_STRASSEN); else GO(f16_t, STHIP_WINOGRAD); }
 #undef GO
@@ -1208,26 +1176,25 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
 }
 
 static int launch_recombine32(int algo, const void* prod, int64_t p_ps, char* C, int64_t c_rs, int64_t c_bs,
-                              int64_t batch, int64_t Mh, int64_t Nh, bool accumulate, hipStream_t stream) {
+                              int64_t batch, int64_t Mh, int64_t Nh, bool accumulate, Call& cx) {
     Recombine16Params rp;
     rp.out_f32 = 1;
     rp.prod = prod; rp.p_ps = p_ps; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;
     rp.Mh = (int)Mh; rp.Nh = (int)Nh; rp.accumulate = accumulate ? 1 : 0;
     dim3 grid((unsigned)ceil_div(Mh * (Nh / 4), 256), (unsigned)batch);
-    if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, stream, rp);
-    else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, stream, rp);
+    if (algo == STHIP_STRASSEN) hipLaunchKernelGGL(recombine32_kernel<STHIP_STRASSEN>, grid, dim3(256), 0, cx.stream, rp);
+    else hipLaunchKernelGGL(recombine32_kernel<STHIP_WINOGRAD>, grid, dim3(256), 0, cx.stream, rp);
     return check_launch("recombine32");
 }
 
 // Two levels of fp32 operands in the same three-launch form (two Strassen levels, nothing
-// rounded; stage-mask bits 4 and 5 off: the five launches sums 1, sums 2, GEMM, 49 -> 7, 7 -> C,
-// which give the same bits): worth it when
+// rounded): worth it when
 // the 49 quarter-size products fill the chip with 256 x 256 tiles, because the seven children
 // of the host recursion would each run their own seven products with a partly empty last round.
 static size_t two_level_f32_bytes(int64_t mh, int64_t nh, int64_t kh) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     return 5 * (align256(mh * kh * 4) + align256(kh * nh * 4)) + 35 * (align256(mq * kq * 4) + align256(kq * nq * 4)) +
-           49 * align256(mq * nq * 4) + 7 * align256(mh * nh * 4);
+           49 * align256(mq * nq * 4);
 }
 
 static bool two_level_f32_shape(int64_t mh, int64_t nh, int64_t kh) {
@@ -1237,50 +1204,28 @@ static bool two_level_f32_shape(int64_t mh, int64_t nh, int64_t kh) {
 }
 
 static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh, int64_t nh, int64_t kh,
-                              bool accumulate, char* ws, hipStream_t stream) {
+                              bool accumulate, char* ws, Call& cx) {
     const int64_t mq = mh / 2, nq = nh / 2, kq = kh / 2;
     const size_t sa1 = align256(mh * kh * 4), sb1 = align256(kh * nh * 4);
     const size_t sa2 = align256(mq * kq * 4), sb2 = align256(kq * nq * 4);
-    const size_t pb = align256(mq * nq * 4), mb = align256(mh * nh * 4);
+    const size_t pb = align256(mq * nq * 4);
     char* SA1 = ws;
     char* SB1 = SA1 + 5 * sa1;
     char* SA2 = SB1 + 5 * sb1;
     char* SB2 = SA2 + 35 * sa2;
     char* P = SB2 + 35 * sb2;
-    char* Mp = P + 49 * pb;
     const bool b_kc = B.rs == 1;
-    const bool fused = (g_stages & 32) != 0;   // sums of both levels in one pass, as for 16-bit operands
-    if (fused) {
+    {
         Combo2Pair pp;
         const int64_t na = fill_combo2(pp.side[0], A, mq, kq, SA1, sa1, SA2, sa2, 0, STHIP_STRASSEN, 4);
         const int64_t nb = fill_combo2(pp.side[1], B, kq, nq, SB1, sb1, SB2, sb2, 1, STHIP_STRASSEN, 4);
         dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-        hipLaunchKernelGGL(quad_combos2_kernel<float>, grid, dim3(256), 0, stream, pp);
+        hipLaunchKernelGGL(quad_combos2_kernel<float>, grid, dim3(256), 0, cx.stream, pp);
         int rc = check_launch("quad_combos2 (fp32)");
-        if (rc) return rc;
-    } else {
-        ComboPair pp;
-        const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA1, sa1, 5, kStrA, 4);
-        const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB1, sb1, 5, kStrB, 4);
-        dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
-        int rc = check_launch("quad_combos (fp32, level 1)");
         if (rc) return rc;
     }
     View xa1[7], xb1[7];
     level_operands(STHIP_STRASSEN, A, B, mh, nh, kh, SA1, sa1, SB1, sb1, xa1, xb1, 4);
-    if (!fused) {
-        ComboMany pm;
-        int64_t most = 0;
-        for (int p = 0; p < 7; ++p) {
-            most = std::max(most, fill_combo(pm.side[2 * p], xa1[p], mq, kq, SA2 + (size_t)p * 5 * sa2, sa2, 5, kStrA, 4));
-            most = std::max(most, fill_combo(pm.side[2 * p + 1], xb1[p], kq, nq, SB2 + (size_t)p * 5 * sb2, sb2, 5, kStrB, 4));
-        }
-        dim3 grid((unsigned)ceil_div(most, 256), 1, 14);
-        hipLaunchKernelGGL(quad_combos_many_f32_kernel, grid, dim3(256), 0, stream, pm);
-        int rc = check_launch("quad_combos (fp32, level 2)");
-        if (rc) return rc;
-    }
     Gemm2Params g;
     memset(&g, 0, sizeof(g));
     for (int p = 0; p < 7; ++p) {
@@ -1294,19 +1239,14 @@ static int two_level_flat_f32(View A, View B, char* C, int64_t c_rs, int64_t mh,
     g.Mh = (int)mq; g.Nh = (int)nq; g.Kh = (int)kq;
     g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
     g.out_f32 = 1; g.accumulate = 0; g.nprod = 49; g.group_m = 4;
-    hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, stream);
+    hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, cx.stream);
     if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
-    if (g_stages & 16) {   // 49 -> C in one pass
-        Recombine16Params rp;
-        rp.prod = P; rp.p_ps = (int64_t)(pb / 4); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
-        rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = 1;
-        dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
-        hipLaunchKernelGGL((recombine16x2_kernel<float, STHIP_STRASSEN>), grid, dim3(256), 0, stream, rp);
-        return check_launch("recombine x2 (fp32)");
-    }
-    int rc = launch_recombine32(STHIP_STRASSEN, P, (int64_t)(pb / 4), Mp, nh, (int64_t)(mb / 4), 7, mq, nq, false, stream);
-    if (rc) return rc;
-    return launch_recombine32(STHIP_STRASSEN, Mp, (int64_t)(mb / 4), C, c_rs, 0, 1, mh, nh, accumulate, stream);
+    Recombine16Params rp;
+    rp.prod = P; rp.p_ps = (int64_t)(pb / 4); rp.C = C; rp.c_rs = c_rs; rp.c_bs = 0;
+    rp.Mh = (int)mq; rp.Nh = (int)nq; rp.accumulate = accumulate ? 1 : 0; rp.out_f32 = 1;
+    dim3 grid((unsigned)ceil_div(mq * (nq / kEPT2), 256), 1);
+    hipLaunchKernelGGL((recombine16x2_kernel<float, STHIP_STRASSEN>), grid, dim3(256), 0, cx.stream, rp);
+    return check_launch("recombine x2 (fp32)");
 }
 
 // Vector form of recombine_kernel: four consecutive columns per thread (nh % 4 == 0, C with unit
@@ -1381,7 +1321,7 @@ static int recombine(int out_dt, char* C, int64_t c_rs, int64_t c_cs, const floa
 // of the classical kernel, and one pass recombines the seven fp32 products into C.  Nothing is
 // rounded anywhere, so the result differs from the fused kernel's only by summation order.
 static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 bool accumulate, char* ws, hipStream_t stream) {
+                                 bool accumulate, char* ws, Call& cx) {
     const size_t sa = align256(Mh * Kh * 4), sb = align256(Kh * Nh * 4), sm = align256(Mh * Nh * 4);
     char* OA = ws;
     char* OB = OA + 7 * sa;
@@ -1390,17 +1330,17 @@ static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t 
     const int64_t na = fill_combo(pp.side[0], A, Mh, Kh, OA, sa, 7, kStr7A, 4);
     const int64_t nb = fill_combo(pp.side[1], B, Kh, Nh, OB, sb, 7, kStr7B, 4);
     dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-    hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+    hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, cx.stream, pp);
     int rc = check_launch("quad_combos (fp32)");
     if (rc) return rc;
     // dense operands keep the storage orientation of their source
     const View a = A.cs == 1 ? View{OA, Kh, 1} : View{OA, 1, Mh};
     const View b = B.cs == 1 ? View{OB, Nh, 1} : View{OB, 1, Kh};
     rc = launch_fused(a, b, Mbuf, Nh, 1, 7, (int64_t)(sa / 4), (int64_t)(sb / 4), (int64_t)(sm / 4), Mh, Nh, Kh, 0, 0, 0,
-                      STHIP_F32, true, STHIP_CLASSIC, false, nullptr, 0, stream);
+                      STHIP_F32, true, STHIP_CLASSIC, false, nullptr, 0, cx);
     if (rc) return rc;
     return recombine(STHIP_F32, C, c_rs, 1, reinterpret_cast<const float*>(Mbuf), (int64_t)(sm / 4), Mh, Nh, 2 * Mh, 2 * Nh,
-                     accumulate, stream);
+                     accumulate, cx.stream);
 }
 
 // Strassen product table in the reference's numbering (fixed_strassen.py:88-114):
@@ -1418,19 +1358,19 @@ static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
 // the seven products (raw quadrants read in place) as one grouped launch into seven dense fp32
 // matrices, one recombination pass.  Nothing is rounded anywhere.
 static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
-                                 int algo, bool accumulate, char* ws, hipStream_t stream) {
+                                 int algo, bool accumulate, char* ws, Call& cx) {
     const size_t sa = align256(Mh * Kh * 4), sb = align256(Kh * Nh * 4), sm = align256(Mh * Nh * 4);
     char* SA = ws;
     char* SB = SA + 5 * sa;
     char* Mbuf = SB + 5 * sb;
     const bool strassen = algo == STHIP_STRASSEN;
     const int nout = strassen ? 5 : 4;
-    if (g_stages & 1) {
+    if (cx.stages & 1) {
         ComboPair pp;
         const int64_t na = fill_combo(pp.side[0], A, Mh, Kh, SA, sa, nout, strassen ? kStrA : kWinA, 4);
         const int64_t nb = fill_combo(pp.side[1], B, Kh, Nh, SB, sb, nout, strassen ? kStrB : kWinB, 4);
         dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, cx.stream, pp);
         int rc = check_launch("quad_combos (fp32)");
         if (rc) return rc;
     }
@@ -1444,26 +1384,28 @@ static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t 
     g.Mh = (int)Mh; g.Nh = (int)Nh; g.Kh = (int)Kh;
     g.tiles_m = (int)(Mh / kBM4); g.tiles_n = (int)(Nh / kBN4);
     g.out_f32 = 1; g.accumulate = 0; g.group_m = 4; g.nprod = 7;
-    if (g_stages & 2) {
-        hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, stream);
+    if (cx.stages & 2) {
+        hipError_t e = table4_for(STHIP_F32)->fn[b_kc ? 1 : 0](g, 1, cx.stream);
         if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
     }
-    if (!(g_stages & 4)) return STHIP_OK;
-    return launch_recombine32(algo, Mbuf, (int64_t)(sm / 4), C, c_rs, 0, 1, Mh, Nh, accumulate, stream);
+    if (!(cx.stages & 4)) return STHIP_OK;
+    return launch_recombine32(algo, Mbuf, (int64_t)(sm / 4), C, c_rs, 0, 1, Mh, Nh, accumulate, cx);
 }
 
-static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels) {
+// inner: the product is one of the seven of an upper level, which takes it in fp32 (16-bit operands
+// then keep their seven products in fp32 too: twice the room).
+static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels, bool inner = false) {
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
     if (levels <= 0) return 0;
     if (levels == 1) {
-        if (fast_shape(dt, mh, nh, kh)) return prepass_bytes(1, mh, nh, kh);
+        if (fast_shape(dt, mh, nh, kh)) return prepass_bytes(1, mh, nh, kh, inner ? 4 : 2);
         if (dt == STHIP_F32 && mh > 0 && nh > 0 && kh > 0 && mh % kBM == 0 && nh % kBN == 0 && kh % 32 == 0)
             return f32_batched_bytes(mh, nh, kh);
         return 0;
     }
     const size_t es = elem_size(dt);
     const size_t recursive = 5 * (align256(mh * kh * es) + align256(kh * nh * es)) + 7 * align256(mh * nh * 4) +
-                             workspace_for(mh, nh, kh, dt, levels - 1);
+                             workspace_for(mh, nh, kh, dt, levels - 1, true);
     // two levels may run as one 49-product launch (two_level_flat) or, if the call's layout or
     // result type rules that out, as the host recursion: room for either
     if (levels == 2 && two_level_shape(dt, mh, nh, kh)) return std::max(recursive, two_level_bytes(mh, nh, kh));
@@ -1476,29 +1418,29 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
 static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                     int64_t M, int64_t N, int64_t K, int64_t Mp, int64_t Np, int64_t Kp,
                     int dt, int out_dt, int algo, int levels, bool accumulate,
-                    char* ws, size_t ws_bytes, hipStream_t stream, bool inner = false) {
+                    char* ws, size_t ws_bytes, Call& cx, bool inner = false) {
     // inner: this product is one of the seven of an upper level, which wants it in fp32; it may
     // still be formed from 16-bit sub-products (only the last rounding is skipped).
     const bool out_f32 = out_dt == STHIP_F32;
     if (algo == STHIP_CLASSIC || levels <= 0)
         return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, 0, 0, 0, dt, out_f32, STHIP_CLASSIC, accumulate,
-                            nullptr, 0, stream);
+                            nullptr, 0, cx);
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
     if (levels == 1)
         return launch_fused(A, B, C, c_rs, c_cs, 1, 0, 0, 0, M, N, K, mh, nh, kh, dt, out_f32, algo, accumulate,
-                            ws, ws_bytes, stream);
+                            ws, ws_bytes, cx);
 
     const size_t es = elem_size(dt);
-    if (levels == 2 && (g_stages & 8) && two_level_shape(dt, mh, nh, kh) && (!out_f32 || inner) && M == Mp && N == Np && K == Kp &&
+    if (levels == 2 && (cx.stages & 8) && two_level_shape(dt, mh, nh, kh) && (!out_f32 || inner) && M == Mp && N == Np && K == Kp &&
         c_cs == 1 && c_rs % 8 == 0 && aligned_to(C, 16) && combos_ok(A, mh, kh) && combos_ok(B, kh, nh) &&
         (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1) && ws && aligned_to(ws, 256) &&
         ws_bytes >= two_level_bytes(mh, nh, kh))
-        return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, stream);
-    if (levels == 2 && (g_stages & 8) && dt == STHIP_F32 && algo == STHIP_STRASSEN && two_level_f32_shape(mh, nh, kh) &&
+        return two_level_flat(A, B, C, c_rs, mh, nh, kh, dt, algo, accumulate, out_f32, ws, cx);
+    if (levels == 2 && (cx.stages & 8) && dt == STHIP_F32 && algo == STHIP_STRASSEN && two_level_f32_shape(mh, nh, kh) &&
         M == Mp && N == Np && K == Kp && c_cs == 1 && c_rs % 4 == 0 && aligned_to(C, 16) && A.cs == 1 &&
         combos_ok(A, mh, kh, 4) && combos_ok(B, kh, nh, 4) && ws && aligned_to(ws, 256) &&
         ws_bytes >= two_level_f32_bytes(mh, nh, kh))
-        return two_level_flat_f32(A, B, C, c_rs, mh, nh, kh, accumulate, ws, stream);
+        return two_level_flat_f32(A, B, C, c_rs, mh, nh, kh, accumulate, ws, cx);
     // Whole, aligned problems: all five sums of each operand in one bandwidth-bound launch.
     const bool whole = M == Mp && N == Np && K == Kp;
     const bool vec = whole && combos_ok(A, mh, kh, (int)es) && combos_ok(B, kh, nh, (int)es);
@@ -1510,10 +1452,12 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     char* SB = ws + 5 * sa_b;
     char* Mbuf = ws + 5 * (sa_b + sb_b);
     char* child_ws = ws + need;
-    const size_t child_bytes = ws_bytes - need;
+    // exactly what the query reserves for a child, however much more the caller passed: the kernels a
+    // child picks depend on the room it is given
+    const size_t child_bytes = std::min(ws_bytes - need, workspace_for(mh, nh, kh, dt, levels - 1, true));
     // B-side sums of this level and of the levels below formed ahead of the call: read, never written
     const char* ready = vec && es == 2 && algo == STHIP_STRASSEN && levels >= 3 && B.rs == 1
-                            ? take_prepared(B.p, levels, kh, nh, prepared_bytes(levels, kh, nh)) : nullptr;
+                            ? take_prepared(cx, B.p, levels, kh, nh, prepared_bytes(levels, kh, nh)) : nullptr;
     const size_t child_prep = ready ? prepared_bytes(levels - 1, kh / 2, nh / 2) : 0;
     if (ready) SB = const_cast<char*>(ready);
 
@@ -1522,13 +1466,13 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         const int64_t na = fill_combo(pp.side[0], A, mh, kh, SA, sa_b, 5, kStrA, 4);
         const int64_t nb = fill_combo(pp.side[1], B, kh, nh, SB, sb_b, 5, kStrB, 4);
         dim3 grid((unsigned)ceil_div(std::max(na, nb), 256), 1, 2);
-        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, stream, pp);
+        hipLaunchKernelGGL(quad_combos_pair_f32_kernel, grid, dim3(256), 0, cx.stream, pp);
         int rc = check_launch("quad_combos (fp32)");
         if (rc) return rc;
     } else if (vec) {
-        int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, stream);
+        int rc = run_combos(dt, A, mh, kh, SA, sa_b, 5, kStrA, cx);
         if (rc) return rc;
-        if (!ready) rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, stream);
+        if (!ready) rc = run_combos(dt, B, kh, nh, SB, sb_b, 5, kStrB, cx);
         if (rc) return rc;
     }
 
@@ -1543,7 +1487,7 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             const char* p = SA + (size_t)kSumA[q] * sa_b;   // dense, in A's storage orientation
             a = A.cs == 1 ? View{p, kh, 1} : View{p, 1, mh};
         } else {
-            int rc = block_sum(dt, SA, A, ara, aca, (ta.b >> 1) * (int)mh, (ta.b & 1) * (int)kh, ta.sign, mh, kh, M, K, stream);
+            int rc = block_sum(dt, SA, A, ara, aca, (ta.b >> 1) * (int)mh, (ta.b & 1) * (int)kh, ta.sign, mh, kh, M, K, cx.stream);
             if (rc) return rc;
             a = {SA, kh, 1};
         }
@@ -1554,22 +1498,22 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             const char* p = SB + (size_t)kSumB[q] * sb_b;
             b = B.cs == 1 ? View{p, nh, 1} : View{p, 1, kh};
         } else {
-            int rc = block_sum(dt, SB, B, bra, bca, (tb.b >> 1) * (int)kh, (tb.b & 1) * (int)nh, tb.sign, kh, nh, K, N, stream);
+            int rc = block_sum(dt, SB, B, bra, bca, (tb.b >> 1) * (int)kh, (tb.b & 1) * (int)nh, tb.sign, kh, nh, K, N, cx.stream);
             if (rc) return rc;
             b = {SB, nh, 1};
         }
-        const PreparedSums outer = g_prep;
+        // the child writes an fp32 product, never the caller's C: no bias for it, and only the sums of its own B operand
+        Call child;
+        child.stream = cx.stream; child.stages = cx.stages; child.force_tile = cx.force_tile;
         if (ready) {
-            g_prep = PreparedSums{};
-            g_prep.sums = ready + 5 * sb_b + (size_t)q * child_prep; g_prep.bytes = child_prep; g_prep.target = b.p;
-            g_prep.levels = levels - 1; g_prep.kh = kh / 2; g_prep.nh = nh / 2;
+            child.prep.sums = ready + 5 * sb_b + (size_t)q * child_prep; child.prep.bytes = child_prep; child.prep.target = b.p;
+            child.prep.levels = levels - 1; child.prep.kh = kh / 2; child.prep.nh = nh / 2;
         }
         int rc = multiply(a, b, Mbuf + q * m_b, nh, 1, mh, nh, kh, mh, nh, kh, dt, STHIP_F32, algo, levels - 1,
-                          false, child_ws, child_bytes, stream, true);
-        g_prep = outer;
+                          false, child_ws, child_bytes, child, true);
         if (rc) return rc;
     }
-    return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, stream);
+    return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, cx.stream);
 }
 
 static int check_common(const void* A, const void* B, const void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
@@ -1611,22 +1555,23 @@ static int static_scratch(char** out) {
     return STHIP_OK;
 }
 
-}  // namespace sthip
-
-using namespace sthip;
-
-extern "C" {
-
-int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
-               const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
-               int in_dtype, int out_dtype, int algo, int levels, int accumulate,
-               void* workspace, size_t workspace_bytes, void* stream) {
+static Call begin_call(void* stream) {
     g_err[0] = 0;
+    Call cx;
+    cx.stream = reinterpret_cast<hipStream_t>(stream);
+    cx.stages = g_debug_stages.load(std::memory_order_relaxed);
+    cx.force_tile = forced_tile_setting();
+    return cx;
+}
+
+static int gemm_impl(Call& cx, const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                     const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
+                     int in_dtype, int out_dtype, int algo, int levels, int accumulate,
+                     void* workspace, size_t workspace_bytes) {
     int rc = check_common(A, B, C, batch, M, N, K, in_dtype, out_dtype, algo, levels);
     if (rc) return rc;
     if (!sA || !sB || !sC) return fail(STHIP_ERR_ARG, "null stride array");
     if (batch == 0 || M == 0 || N == 0) return STHIP_OK;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const int es = elem_size(in_dtype), ces = elem_size(out_dtype);
     if (algo == STHIP_CLASSIC) levels = 0;
     if (algo != STHIP_CLASSIC && levels == 0) algo = STHIP_CLASSIC;
@@ -1637,23 +1582,108 @@ int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, 
         View b = {reinterpret_cast<const char*>(B), sB[1], sB[2]};
         return launch_fused(a, b, reinterpret_cast<char*>(C), sC[1], sC[2], batch, sA[0], sB[0], sC[0], M, N, K,
                             Mp / 2, Np / 2, Kp / 2, in_dtype, out_dtype == STHIP_F32, algo, accumulate != 0,
-                            reinterpret_cast<char*>(workspace), workspace_bytes, s);
+                            reinterpret_cast<char*>(workspace), workspace_bytes, cx);
     }
     for (int64_t bi = 0; bi < batch; ++bi) {
         View a = {reinterpret_cast<const char*>(A) + bi * sA[0] * es, sA[1], sA[2]};
         View b = {reinterpret_cast<const char*>(B) + bi * sB[0] * es, sB[1], sB[2]};
         char* c = reinterpret_cast<char*>(C) + bi * sC[0] * ces;
         rc = multiply(a, b, c, sC[1], sC[2], M, N, K, Mp, Np, Kp, in_dtype, out_dtype, algo, levels, accumulate != 0,
-                      reinterpret_cast<char*>(workspace), workspace_bytes, s);
+                      reinterpret_cast<char*>(workspace), workspace_bytes, cx);
         if (rc) return rc;
     }
     return STHIP_OK;
 }
 
+// The bias of a Linear forward goes into the last pass of the product where that pass can take it
+// (16-bit, 16-byte aligned); otherwise a pass of its own adds it afterwards.
+static void offer_bias(Call& cx, const void* bias, const void* y, int dtype) {
+    cx.bias = BiasEpilogue{};
+    if (bias && dtype != STHIP_F32 && aligned_to(bias, 16)) { cx.bias.bias = bias; cx.bias.target = y; }
+}
+static int finish_bias(Call& cx, const void* bias, void* y, int64_t rows, int64_t cols, int dtype) {
+    if (!bias || cx.bias.applied) return STHIP_OK;
+    const unsigned blocks = (unsigned)ceil_div(rows * cols, 256);
+    char* yy = reinterpret_cast<char*>(y);
+    const char* bb = reinterpret_cast<const char*>(bias);
+    if (dtype == STHIP_F32) hipLaunchKernelGGL(add_bias_kernel<float>, dim3(blocks), dim3(256), 0, cx.stream, yy, bb, rows, cols);
+    else if (dtype == STHIP_F16) hipLaunchKernelGGL(add_bias_kernel<f16_t>, dim3(blocks), dim3(256), 0, cx.stream, yy, bb, rows, cols);
+    else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3(blocks), dim3(256), 0, cx.stream, yy, bb, rows, cols);
+    return check_launch("add_bias");
+}
+
+static int linear_forward_impl(Call& cx, const void* x, const void* W, const void* bias, void* y,
+                               int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
+                               void* workspace, size_t workspace_bytes) {
+    int rc = check_common(x, W, y, 1, rows, out_features, in_features, dtype, dtype, STHIP_STRASSEN, levels);
+    if (rc) return rc;
+    if (rows == 0 || out_features == 0) return STHIP_OK;
+    const int64_t sA[3] = {0, in_features, 1}, sB[3] = {0, 1, in_features}, sC[3] = {0, out_features, 1};   // B = W^T as a view
+    offer_bias(cx, bias, y, dtype);
+    rc = gemm_impl(cx, x, W, y, 1, rows, out_features, in_features, sA, sB, sC, dtype, dtype,
+                   levels > 0 ? STHIP_STRASSEN : STHIP_CLASSIC, levels, 0, workspace, workspace_bytes);
+    if (rc) return rc;
+    return finish_bias(cx, bias, y, rows, out_features, dtype);
+}
+
+// Half extents of W^T (in_features x out_features) for which the weight-side sums can be formed
+// ahead of the call: 16-bit operands, one to four levels, innermost blocks that the grouped paths take.
+static bool weight_sums_shape(int64_t in_features, int64_t out_features, int dtype, int levels) {
+    if (dtype != STHIP_BF16 && dtype != STHIP_F16) return false;
+    if (levels < 1 || levels > 4) return false;
+    const int64_t q = (int64_t)1 << levels;
+    if (in_features <= 0 || out_features <= 0 || in_features % q || out_features % q) return false;
+    return fast_shape(dtype, 128, out_features / q, in_features / q);
+}
+
+// Sums of the k x n operand B (stored n-major: B.rs == 1) for `levels` levels into `buf`.
+static int prepare_b(int dt, View B, int64_t k, int64_t n, int levels, char* buf, Call& cx) {
+    const int64_t kh = k / 2, nh = n / 2;
+    const size_t sb1 = align256(kh * nh * 2);
+    if (levels == 1) return run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, cx);
+    if (levels == 2) {
+        const size_t sb2 = align256((kh / 2) * (nh / 2) * 2);
+        Combo2Pair pp;
+        memset(&pp, 0, sizeof(pp));
+        const int64_t nb = fill_combo2(pp.side[0], B, kh / 2, nh / 2, buf, sb1, buf + 5 * sb1, sb2, 1, STHIP_STRASSEN);
+        dim3 grid((unsigned)ceil_div(nb, 256), 1, 1);
+        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, cx.stream, pp);
+        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, cx.stream, pp);
+        return check_launch("quad_combos2 (weight)");
+    }
+    int rc = run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, cx);
+    if (rc) return rc;
+    const size_t child = prepared_bytes(levels - 1, kh / 2, nh / 2);
+    for (int q = 0; q < 7; ++q) {
+        // B operand of product M(q+1) as multiply() forms it: a quadrant in place or a dense sum
+        const Term tb = kBTerms[q];
+        const View b = tb.sign == 0 ? View{B.p + ((int64_t)(tb.a >> 1) * kh * B.rs + (int64_t)(tb.a & 1) * nh * B.cs) * 2, B.rs, B.cs}
+                                    : View{buf + (size_t)kSumB[q] * sb1, 1, kh};
+        rc = prepare_b(dt, b, kh, nh, levels - 1, buf + 5 * sb1 + (size_t)q * child, cx);
+        if (rc) return rc;
+    }
+    return STHIP_OK;
+}
+
+}  // namespace sthip
+
+using namespace sthip;
+
+extern "C" {
+
+int sthip_gemm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+               const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
+               int in_dtype, int out_dtype, int algo, int levels, int accumulate,
+               void* workspace, size_t workspace_bytes, void* stream) {
+    Call cx = begin_call(stream);
+    return gemm_impl(cx, A, B, C, batch, M, N, K, sA, sB, sC, in_dtype, out_dtype, algo, levels, accumulate,
+                     workspace, workspace_bytes);
+}
+
 int sthip_gemm_static(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
                       const int64_t sA[3], const int64_t sB[3], const int64_t sC[3],
                       int in_dtype, int out_dtype, int algo, int levels, int accumulate, void* stream) {
-    g_err[0] = 0;
+    Call cx = begin_call(stream);
     int rc = check_common(A, B, C, batch, M, N, K, in_dtype, out_dtype, algo, levels);
     if (rc) return rc;
     const size_t need = sthip_workspace_bytes(batch, M, N, K, in_dtype, out_dtype, algo, levels);
@@ -1665,7 +1695,7 @@ int sthip_gemm_static(const void* A, const void* B, void* C, int64_t batch, int6
         rc = static_scratch(&ws);
         if (rc) return rc;
     }
-    return sthip_gemm(A, B, C, batch, M, N, K, sA, sB, sC, in_dtype, out_dtype, algo, levels, accumulate, ws, need, stream);
+    return gemm_impl(cx, A, B, C, batch, M, N, K, sA, sB, sC, in_dtype, out_dtype, algo, levels, accumulate, ws, need);
 }
 
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {
@@ -1688,89 +1718,46 @@ size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int
 int sthip_strassen_matmul_n_layers(const void* A, const void* B, void* C, int64_t n,
                                    int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs,
                                    int dtype, int levels, void* workspace, size_t workspace_bytes, void* stream) {
+    Call cx = begin_call(stream);
     const int64_t sA[3] = {0, a_rs, a_cs}, sB[3] = {0, b_rs, b_cs}, sC[3] = {0, n, 1};
     if (levels < 1) return fail(STHIP_ERR_ARG, "levels must be >= 1, got %d", levels);
-    return sthip_gemm(A, B, C, 1, n, n, n, sA, sB, sC, dtype, dtype, STHIP_STRASSEN, levels, 0, workspace, workspace_bytes, stream);
+    return gemm_impl(cx, A, B, C, 1, n, n, n, sA, sB, sC, dtype, dtype, STHIP_STRASSEN, levels, 0, workspace, workspace_bytes);
 }
 
 int sthip_run_accumulate(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
                          int op_dtype, int c_dtype, int algo, int levels,
                          void* workspace, size_t workspace_bytes, void* stream) {
+    Call cx = begin_call(stream);
     const int64_t sA[3] = {M * K, K, 1}, sB[3] = {K * N, N, 1}, sC[3] = {M * N, N, 1};
-    return sthip_gemm(A, B, C, batch, M, N, K, sA, sB, sC, op_dtype, c_dtype, algo, levels, 1, workspace, workspace_bytes, stream);
+    return gemm_impl(cx, A, B, C, batch, M, N, K, sA, sB, sC, op_dtype, c_dtype, algo, levels, 1, workspace, workspace_bytes);
 }
 
 int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias, void* y,
                                   int64_t rows, int64_t D, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream) {
-    g_err[0] = 0;
+    Call cx = begin_call(stream);
     int rc = check_common(x, W, y, 1, rows, D, D, dtype, dtype, STHIP_STRASSEN, levels);
     if (rc) return rc;
     if (levels < 1) return fail(STHIP_ERR_ARG, "levels must be >= 1, got %d", levels);
     if (rows > D) return fail(STHIP_ERR_SHAPE, "rows (%lld) > D (%lld): the input cannot be padded to D x D", (long long)rows, (long long)D);
     if (rows == 0 || D == 0) return STHIP_OK;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     // The reference pads x to D x D (model/layers.py:261-262): split on the padded size.
     const int64_t q = (int64_t)1 << levels;
     const int64_t Dp = round_up(D, q);
     View a = {reinterpret_cast<const char*>(x), D, 1};
     View b = {reinterpret_cast<const char*>(W), 1, D};   // W^T as a view
-    g_bias = BiasEpilogue{};
-    if (bias && dtype != STHIP_F32 && reinterpret_cast<uintptr_t>(bias) % 16 == 0) { g_bias.bias = bias; g_bias.target = y; }
+    offer_bias(cx, bias, y, dtype);
     rc = multiply(a, b, reinterpret_cast<char*>(y), D, 1, rows, D, D, Dp, Dp, Dp, dtype, dtype, STHIP_STRASSEN, levels, false,
-                  reinterpret_cast<char*>(workspace), workspace_bytes, s);
-    const bool bias_done = g_bias.applied;
-    g_bias = BiasEpilogue{};
+                  reinterpret_cast<char*>(workspace), workspace_bytes, cx);
     if (rc) return rc;
-    if (bias && !bias_done) {
-        const int64_t n = rows * D;
-        const unsigned blocks = (unsigned)ceil_div(n, 256);
-        char* yy = reinterpret_cast<char*>(y);
-        const char* bb = reinterpret_cast<const char*>(bias);
-        if (dtype == STHIP_F32) hipLaunchKernelGGL(add_bias_kernel<float>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
-        else if (dtype == STHIP_F16) hipLaunchKernelGGL(add_bias_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
-        else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, D);
-        return check_launch("add_bias");
-    }
-    return STHIP_OK;
+    return finish_bias(cx, bias, y, rows, D, dtype);
 }
 
 int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y,
                          int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                          void* workspace, size_t workspace_bytes, void* stream) {
-    g_err[0] = 0;
-    int rc = check_common(x, W, y, 1, rows, out_features, in_features, dtype, dtype, STHIP_STRASSEN, levels);
-    if (rc) return rc;
-    if (rows == 0 || out_features == 0) return STHIP_OK;
-    const int64_t sA[3] = {0, in_features, 1}, sB[3] = {0, 1, in_features}, sC[3] = {0, out_features, 1};   // B = W^T as a view
-    g_bias = BiasEpilogue{};
-    if (bias && dtype != STHIP_F32 && reinterpret_cast<uintptr_t>(bias) % 16 == 0) { g_bias.bias = bias; g_bias.target = y; }
-    rc = sthip_gemm(x, W, y, 1, rows, out_features, in_features, sA, sB, sC, dtype, dtype,
-                    levels > 0 ? STHIP_STRASSEN : STHIP_CLASSIC, levels, 0, workspace, workspace_bytes, stream);
-    const bool bias_done = g_bias.applied;
-    g_bias = BiasEpilogue{};
-    if (rc) return rc;
-    if (bias && !bias_done) {
-        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-        const unsigned blocks = (unsigned)ceil_div(rows * out_features, 256);
-        char* yy = reinterpret_cast<char*>(y);
-        const char* bb = reinterpret_cast<const char*>(bias);
-        if (dtype == STHIP_F32) hipLaunchKernelGGL(add_bias_kernel<float>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
-        else if (dtype == STHIP_F16) hipLaunchKernelGGL(add_bias_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
-        else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, yy, bb, rows, out_features);
-        return check_launch("add_bias");
-    }
-    return STHIP_OK;
-}
-
-// Half extents of W^T (in_features x out_features) for which the weight-side sums can be formed
-// ahead of the call: 16-bit operands, one to four levels, innermost blocks that the grouped paths take.
-static bool weight_sums_shape(int64_t in_features, int64_t out_features, int dtype, int levels) {
-    if (dtype != STHIP_BF16 && dtype != STHIP_F16) return false;
-    if (levels < 1 || levels > 4) return false;
-    const int64_t q = (int64_t)1 << levels;
-    if (in_features <= 0 || out_features <= 0 || in_features % q || out_features % q) return false;
-    return fast_shape(dtype, 128, out_features / q, in_features / q);
+    Call cx = begin_call(stream);
+    return linear_forward_impl(cx, x, W, bias, y, rows, in_features, out_features, dtype, levels, workspace, workspace_bytes);
 }
 
 size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features, int dtype, int levels) {
@@ -1778,38 +1765,9 @@ size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features,
     return prepared_bytes(levels, in_features / 2, out_features / 2);
 }
 
-// Sums of the k x n operand B (stored n-major: B.rs == 1) for `levels` levels into `buf`.
-static int prepare_b(int dt, View B, int64_t k, int64_t n, int levels, char* buf, hipStream_t s) {
-    const int64_t kh = k / 2, nh = n / 2;
-    const size_t sb1 = align256(kh * nh * 2);
-    if (levels == 1) return run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, s);
-    if (levels == 2) {
-        const size_t sb2 = align256((kh / 2) * (nh / 2) * 2);
-        Combo2Pair pp;
-        memset(&pp, 0, sizeof(pp));
-        const int64_t nb = fill_combo2(pp.side[0], B, kh / 2, nh / 2, buf, sb1, buf + 5 * sb1, sb2, 1, STHIP_STRASSEN);
-        dim3 grid((unsigned)ceil_div(nb, 256), 1, 1);
-        if (dt == STHIP_BF16) hipLaunchKernelGGL(quad_combos2_kernel<bf16_t>, grid, dim3(256), 0, s, pp);
-        else hipLaunchKernelGGL(quad_combos2_kernel<f16_t>, grid, dim3(256), 0, s, pp);
-        return check_launch("quad_combos2 (weight)");
-    }
-    int rc = run_combos(dt, B, kh, nh, buf, sb1, 5, kStrB, s);
-    if (rc) return rc;
-    const size_t child = prepared_bytes(levels - 1, kh / 2, nh / 2);
-    for (int q = 0; q < 7; ++q) {
-        // B operand of product M(q+1) as multiply() forms it: a quadrant in place or a dense sum
-        const Term tb = kBTerms[q];
-        const View b = tb.sign == 0 ? View{B.p + ((int64_t)(tb.a >> 1) * kh * B.rs + (int64_t)(tb.a & 1) * nh * B.cs) * 2, B.rs, B.cs}
-                                    : View{buf + (size_t)kSumB[q] * sb1, 1, kh};
-        rc = prepare_b(dt, b, kh, nh, levels - 1, buf + 5 * sb1 + (size_t)q * child, s);
-        if (rc) return rc;
-    }
-    return STHIP_OK;
-}
-
 int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_features, int dtype, int levels,
                                 void* sums, size_t sums_bytes, void* stream) {
-    g_err[0] = 0;
+    Call cx = begin_call(stream);
     const size_t need = sthip_linear_weight_sums_bytes(in_features, out_features, dtype, levels);
     if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d (16-bit, 1 to 4 levels, aligned blocks)",
                            (long long)in_features, (long long)out_features, dtype, levels);
@@ -1817,37 +1775,34 @@ int sthip_linear_prepare_weight(const void* W, int64_t in_features, int64_t out_
     if (!aligned_to(W, 16)) return fail(STHIP_ERR_ARG, "W must be 16-byte aligned");
     if (!aligned_to(sums, 256)) return fail(STHIP_ERR_ARG, "the sums buffer must be 256-byte aligned");
     if (sums_bytes < need) return fail(STHIP_ERR_WORKSPACE, "sums buffer too small: %zu < %zu bytes", sums_bytes, need);
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const View B = {reinterpret_cast<const char*>(W), 1, in_features};   // W^T as a view
-    return prepare_b(dtype, B, in_features, out_features, levels, reinterpret_cast<char*>(sums), s);
+    return prepare_b(dtype, B, in_features, out_features, levels, reinterpret_cast<char*>(sums), cx);
 }
 
 int sthip_linear_forward_prepared(const void* x, const void* W, const void* sums, size_t sums_bytes, const void* bias, void* y,
                                   int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream) {
-    g_err[0] = 0;
+    Call cx = begin_call(stream);
     const size_t need = sthip_linear_weight_sums_bytes(in_features, out_features, dtype, levels);
     if (!need) return fail(STHIP_ERR_SHAPE, "no weight-side sums for in=%lld out=%lld dtype=%d levels=%d",
                            (long long)in_features, (long long)out_features, dtype, levels);
     if (!sums || !aligned_to(sums, 256)) return fail(STHIP_ERR_ARG, "the sums buffer must be non-null and 256-byte aligned");
     if (sums_bytes < need) return fail(STHIP_ERR_WORKSPACE, "sums buffer too small: %zu < %zu bytes", sums_bytes, need);
-    g_prep = PreparedSums{};
-    g_prep.sums = reinterpret_cast<const char*>(sums); g_prep.bytes = sums_bytes; g_prep.target = W;
-    g_prep.levels = levels; g_prep.kh = in_features / 2; g_prep.nh = out_features / 2;
-    const int rc = sthip_linear_forward(x, W, bias, y, rows, in_features, out_features, dtype, levels, workspace, workspace_bytes, stream);
-    g_prep = PreparedSums{};
-    return rc;
-}
-
-int sthip_debug_set_stages(int mask) {
-    const int old = g_stages;
-    g_stages = mask & 63;
-    return old;
+    cx.prep.sums = reinterpret_cast<const char*>(sums); cx.prep.bytes = sums_bytes; cx.prep.target = W;
+    cx.prep.levels = levels; cx.prep.kh = in_features / 2; cx.prep.nh = out_features / 2;
+    return linear_forward_impl(cx, x, W, bias, y, rows, in_features, out_features, dtype, levels, workspace, workspace_bytes);
 }
 
 const char* sthip_last_error(void) { return g_err; }
 
 int sthip_version(void) { return STHIP_VERSION; }
+
+int sthip_debug_set_stages(int mask) { return g_debug_stages.exchange(mask & kAllStages); }
+
+int sthip_debug_force_tile(const char* tile) {
+    forced_tile_setting();   // settle the environment's value first, so that it cannot overwrite this one later
+    return g_debug_tile.exchange(tile_code(tile));
+}
 
 int sthip_debug_transpose_read(void* out, void* stream) {
     g_err[0] = 0;

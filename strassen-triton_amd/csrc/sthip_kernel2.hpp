@@ -24,13 +24,6 @@
 
 namespace sthip {
 
-// Experiment switches for kernel4_microbench.hip (always 0 in the library):
-// 1 = skip the global->LDS loads, 2 = skip the workgroup barrier, 4 = skip the fragment reads,
-// 64 = skip the MFMAs.
-#ifndef STHIP_DBG
-#define STHIP_DBG 0
-#endif
-
 constexpr int kMaxSeg = 49;   // seven products of one level, or the 49 of two levels in one launch
 constexpr int kStages = 4;
 constexpr int kBK2 = 64;                       // k per step (16-bit operands)
@@ -203,22 +196,19 @@ struct Pipe2 {
                     // Next stage must be visible to everyone before its fragments are read; this
                     // barrier also retires stage g-1, whose buffer the next load reuses.
                     const int ahead = total - 1 - g;        // steps after this one
-                    if (!(STHIP_DBG & 1)) { if (ahead >= 2) wait_vmcnt(8); else wait_vmcnt(0); }
-                    if (!(STHIP_DBG & 2)) __syncthreads();
-                    if (!(STHIP_DBG & 1) && !ld.done()) ld.issue(stage_addr(g + kStages - 1));
+                    if (ahead >= 2) wait_vmcnt(8); else wait_vmcnt(0);
+                    __syncthreads();
+                    if (!ld.done()) ld.issue(stage_addr(g + kStages - 1));
                 }
                 const int nb = (kg + 1) & 1;
-                if (!(STHIP_DBG & 4)) {
-                    if (kg < 3) read_frags(nb, g, kg + 1);
-                    else if (g + 1 < total) read_frags(nb, g + 1, 0);
-                }
+                if (kg < 3) read_frags(nb, g, kg + 1);
+                else if (g + 1 < total) read_frags(nb, g + 1, 0);
                 const int cb = kg & 1;
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        if (!(STHIP_DBG & 64)) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
-                        else acc.t[i][j][0] += __builtin_bit_cast(float, fa[cb][i][0] ^ fb[cb][j][0]);   // experiment: no MFMA
+                        mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                     }
             }
         }

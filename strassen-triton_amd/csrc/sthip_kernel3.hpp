@@ -79,14 +79,10 @@ struct Loader3 {
         const uint32_t sa = stage_addr + wave * 8192, sb = stage_addr + kATile3 + wave * 4096;
 #pragma unroll
         for (int i = 0; i < 8; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
-        if (!(STHIP_DBG & 16)) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], sb + i * 1024);
-        }
-        if (!(STHIP_DBG & 8)) {
-            a_base += a_step_bytes;
-            b_base += b_step_bytes;
-        }
+        for (int i = 0; i < 4; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], sb + i * 1024);
+        a_base += a_step_bytes;
+        b_base += b_step_bytes;
         if (++kt == KT) {
             kt = 0;
             if (++seg < total_seg) point_at_segment();
@@ -181,33 +177,30 @@ struct Pipe3 {
             for (int kg = 0; kg < 4; ++kg) {
                 const int nb = (kg + 1) & 1, cb = kg & 1;
                 if (kg < 3) {
-                    if (!(STHIP_DBG & 4)) read_frags(nb, slot, kg + 1);
+                    read_frags(nb, slot, kg + 1);
                 } else {
                     const int ahead = total - 1 - g;   // steps after this one
                     // in flight: step g+1 (needed now) and step g+2
-                    if (!(STHIP_DBG & 1)) { if (ahead >= 2) wait_vmcnt_imm<12>(); else wait_vmcnt_imm<0>(); }
-                    if (!(STHIP_DBG & 2)) __syncthreads();
-                    if (!(STHIP_DBG & 1) && !ld.done()) ld.issue(smem_addr + slot * kStageBytes3);
-                    if (!(STHIP_DBG & 4) && ahead > 0) read_frags(nb, next_slot(slot), 0);
+                    if (ahead >= 2) wait_vmcnt_imm<12>(); else wait_vmcnt_imm<0>();
+                    __syncthreads();
+                    if (!ld.done()) ld.issue(smem_addr + slot * kStageBytes3);
+                    if (ahead > 0) read_frags(nb, next_slot(slot), 0);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        if (!(STHIP_DBG & 64)) mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
-                        else acc.t[i][j][0] += __builtin_bit_cast(float, fa[cb][i][0] ^ fb[cb][j][0]);   // experiment
+                        mfma_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                     }
                 // Pin the software pipeline: the fragment reads of the next k-group are spread one
                 // per MFMA of this k-group, so their LDS latency hides behind matrix-core time
                 // instead of being sunk next to their first use.
-                if (!(STHIP_DBG & 128)) {
 #pragma unroll
-                    for (int m = 0; m < 8; ++m) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int m = 0; m < 8; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
             slot = next_slot(slot);
         }

@@ -117,10 +117,8 @@ struct Loader4 {
         }
     }
     __device__ __forceinline__ void advance() {
-        if (!(STHIP_DBG & 128)) {   // bit 128: every k-step loads the first one again (cache hits)
-            a_base += a_step_bytes;
-            b_base += b_step_bytes;
-        }
+        a_base += a_step_bytes;
+        b_base += b_step_bytes;
         if (++kt == KT) {
             kt = 0;
             if (++seg < total_seg) point_at_segment();
@@ -231,19 +229,11 @@ struct Pipe4 {
     __device__ __forceinline__ void start() {
         g = 0;
         slot = 0;
-        if (STHIP_DBG & 4) {
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) { fa[b][i] = u32x4{0, 0, 0, 0}; fb[b][i & 3] = u32x4{0, 0, 0, 0}; }
-        }
-        if (!(STHIP_DBG & 1)) {
-            ld.issue(smem_addr);
-            if (!ld.done()) ld.issue(smem_addr + kStageBytes4);
-            if (total >= 2) wait_vmcnt_imm<8>(); else wait_vmcnt_imm<0>();   // step 0 has landed
-        }
+        ld.issue(smem_addr);
+        if (!ld.done()) ld.issue(smem_addr + kStageBytes4);
+        if (total >= 2) wait_vmcnt_imm<8>(); else wait_vmcnt_imm<0>();   // step 0 has landed
         __syncthreads();
-        if (!(STHIP_DBG & 4)) read_frags(0, 0, 0);
+        read_frags(0, 0, 0);
     }
 
     __device__ __forceinline__ void run(Acc4& acc, int KT) {
@@ -255,12 +245,12 @@ struct Pipe4 {
                     // Every wave has read all fragments of this step: after the barrier its stage is
                     // free for the step two ahead.  Step g+1 (the only load batch in flight) must
                     // have landed before its fragments are read.
-                    if (!(STHIP_DBG & 1)) wait_vmcnt_imm<0>();
-                    if (!(STHIP_DBG & 2)) __syncthreads();
+                    wait_vmcnt_imm<0>();
+                    __syncthreads();
                 }
                 // The wave's eight loads of step g+2 go out one per row of matrix instructions
                 // (measured at 8192^3: one per row 0.865 ms, two 0.879, four or all at once 0.895).
-                const bool issuing = kg == 1 && !(STHIP_DBG & 1) && !ld.done();
+                const bool issuing = kg == 1 && !ld.done();
                 // Fragments of the next k-group come in between the rows of matrix instructions, one
                 // A and (first four rows) one B fragment per row: few enough in flight for the LDS
                 // counter (4 bits) to tell the old fragments from the new, and bursts of reads cost
@@ -273,9 +263,7 @@ struct Pipe4 {
                         ld.issue_one(smem_addr + slot * kStageBytes4, i);
                         if (i == 7) ld.advance();
                     }
-                    if (!(STHIP_DBG & 4)) {
-                        read_pair(nb, nsl, nkg, i);
-                    }
+                    read_pair(nb, nsl, nkg, i);
                     if constexpr (es4<T>() == 4) {
                         // four matrix instructions per accumulator and k-group: component-major, so
                         // that instructions on one accumulator are four apart
@@ -283,12 +271,12 @@ struct Pipe4 {
                         for (int c = 0; c < 4; ++c)
 #pragma unroll
                             for (int j = 0; j < 4; ++j)
-                                if (!(STHIP_DBG & 64)) mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
+                                mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
                     } else {
 #pragma unroll
                         for (int jj = 0; jj < 4; ++jj) {
                             const int j = (i & 1) ? 3 - jj : jj;   // boustrophedon: the B fragment carries over between rows
-                            if (!(STHIP_DBG & 64)) mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
+                            mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -414,7 +402,6 @@ __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2
 template <class T, bool B_KC>
 __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    if (STHIP_DBG & 16) return;
     // blockIdx.x = product * tiles + tile: the XCD-aware renumbering works within one product
     const int tiles = P.tiles_m * P.tiles_n;
     const int prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
@@ -444,11 +431,10 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     Acc4 r;
     r.zero();
     pipe.run(r, KT);
-    if (STHIP_DBG & 8) return;
-    if (P.c_wide && !P.out_f32 && !P.accumulate && !(STHIP_DBG & 32)) {
+    if (P.c_wide && !P.out_f32 && !P.accumulate) {
         __syncthreads();   // every wave has read its last fragments: the stage buffers are free
         store_tile4_lds<T>(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
-    } else if (P.out_f32 && !P.accumulate && !(STHIP_DBG & 32)) {
+    } else if (P.out_f32 && !P.accumulate) {
         __syncthreads();
         store_tile4_lds_f32(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
     } else {

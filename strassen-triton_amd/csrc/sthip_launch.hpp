@@ -1,6 +1,7 @@
 // Launch table shared by the kernel instantiation units and the C-ABI front end.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include "sthip_kernel.hpp"
 #include "sthip_kernel2.hpp"
 #include "sthip_kernel3.hpp"
@@ -9,6 +10,22 @@
 namespace sthip {
 
 enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+
+// More than 64 KiB of dynamic LDS needs an explicit opt-in per kernel, once per device.  `done` is the
+// kernel's own flag array; two threads that race here both set the (idempotent) attribute.
+struct OptIn { std::atomic<bool> done[64]; };
+inline hipError_t opt_in_lds(OptIn& o, const void* kern, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (!o.done[dev].load(std::memory_order_acquire)) {
+        e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        o.done[dev].store(true, std::memory_order_release);
+    }
+    return hipSuccess;
+}
 
 // One table per (element type, algorithm), indexed [a_kc][b_kc][edge]; each is defined by
 // one compilation of sthip_inst.hip.
@@ -24,16 +41,9 @@ template <class T, int ALGO, bool A_KC, bool B_KC, bool EDGE>
 hipError_t launch_gemm(const GemmParams& p, int batch, hipStream_t stream) {
     using C = Ctx<T, A_KC, B_KC>;
     auto kern = gemm_kernel<T, ALGO, A_KC, B_KC, EDGE>;
-    // More than 64 KiB of dynamic LDS needs an explicit opt-in, once per device.
-    static bool opted[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    static OptIn opted;
+    hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), C::SMEM_BYTES);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES);
-        if (e != hipSuccess) return e;
-        opted[dev] = true;
-    }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads), C::SMEM_BYTES, stream, p);
     return hipGetLastError();
@@ -50,15 +60,9 @@ STHIP_DECLARE_TABLE2(2, 0) STHIP_DECLARE_TABLE2(2, 1) STHIP_DECLARE_TABLE2(2, 2)
 template <class T, int ALGO, bool A_KC, bool B_KC>
 hipError_t launch_gemm2(const Gemm2Params& p, int batch, hipStream_t stream) {
     auto kern = gemm2_kernel<T, ALGO, A_KC, B_KC>;
-    static bool opted[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    static OptIn opted;
+    hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes2);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes2);
-        if (e != hipSuccess) return e;
-        opted[dev] = true;
-    }
     const int nprod = ALGO == ALGO_CLASSIC && p.nprod > 0 ? p.nprod : 1;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads), kSmemBytes2, stream, p);
@@ -75,15 +79,9 @@ STHIP_DECLARE_TABLE3(2, 0) STHIP_DECLARE_TABLE3(2, 1) STHIP_DECLARE_TABLE3(2, 2)
 template <class T, int ALGO, bool B_KC>
 hipError_t launch_gemm3(const Gemm2Params& p, int batch, hipStream_t stream) {
     auto kern = gemm3_kernel<T, ALGO, B_KC>;
-    static bool opted[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    static OptIn opted;
+    hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes3);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes3);
-        if (e != hipSuccess) return e;
-        opted[dev] = true;
-    }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads3), kSmemBytes3, stream, p);
     return hipGetLastError();
@@ -98,15 +96,9 @@ extern const LaunchTable3 kLaunch4_2;
 template <class T, bool B_KC>
 hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
     auto kern = gemm4_kernel<T, B_KC>;
-    static bool opted[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    static OptIn opted;
+    hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes4);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes4);
-        if (e != hipSuccess) return e;
-        opted[dev] = true;
-    }
     const int nprod = p.nprod > 0 ? p.nprod : 1;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, p);

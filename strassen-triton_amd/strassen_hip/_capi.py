@@ -1,4 +1,5 @@
-"""ctypes binding of libstrassen_hip.so (the C ABI declared in include/strassen_hip.h).
+"""ctypes binding of libstrassen_hip.so (the C ABI declared in include/strassen_hip.h, and the
+test hooks of include/strassen_hip_debug.h).
 
 Nothing here falls back to another implementation: if the shared library is missing the
 import of any product module fails with the build command to run.
@@ -11,7 +12,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libstrassen_hip.so")
 
-# name -> (restype, argtypes); must list every symbol include/strassen_hip.h declares
+# name -> (restype, argtypes); must list every symbol the two headers declare
 _i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 _p64 = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
@@ -33,6 +34,7 @@ SIGNATURES = {
     "sthip_version": (_int, []),
     "sthip_debug_transpose_read": (_int, [_vp, _vp]),
     "sthip_debug_set_stages": (_int, [_int]),
+    "sthip_debug_force_tile": (_int, [ctypes.c_char_p]),
 }
 
 _lib = None

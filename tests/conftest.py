@@ -34,3 +34,22 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def force_tile():
+    """force_tile("256x256") overrides the library's tile table (sthip_debug_force_tile) until the
+    test ends; the previous setting comes back afterwards."""
+    from strassen_hip import _capi
+    lib = _capi.load()
+    names = {0: None, 2: b"128x128", 3: b"256x128", 4: b"256x256", 5: b"128x128g"}
+    first = []
+
+    def force(tile):
+        prev = lib.sthip_debug_force_tile(tile.encode() if tile else None)
+        if not first:
+            first.append(prev)
+
+    yield force
+    if first:
+        lib.sthip_debug_force_tile(names[first[0]])

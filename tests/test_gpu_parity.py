@@ -255,12 +255,6 @@ def test_two_levels_as_one_launch(hip, dtype, algo, ta, tb, shape):
         rec = hip.gemm(Ag, Bg, algo=algo, levels=2)
     finally:
         lib.sthip_debug_set_stages(prev)
-    prev = lib.sthip_debug_set_stages(15)   # bit 4 off: 49 -> 7 -> C as two recombination passes
-    try:
-        two_pass = hip.gemm(Ag, Bg, algo=algo, levels=2)
-    finally:
-        lib.sthip_debug_set_stages(prev)
-    assert torch.equal(flat, two_pass)      # the one-pass recombination rounds and adds in the same places
     ref = Ag.double() @ Bg.double()
     rel = lambda X: float(torch.linalg.norm(X.double() - ref) / torch.linalg.norm(ref))
     assert rel(flat) <= TOL[dtype] and rel(rec) <= TOL[dtype]
@@ -289,10 +283,10 @@ def test_three_levels_16bit(hip, dtype, tb):
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 320), (1024, 1024, 1024)])
-def test_fp32_batched_products(hip, monkeypatch, ta, tb, shape):
+def test_fp32_batched_products(hip, force_tile, ta, tb, shape):
     """fp32, one level, tile-aligned: the seven products run as one batched classical launch
     over dense operand copies.  Exact on integers; on random inputs within 1e-5 of fp64 and of
-    the fused kernel (forced with STHIP_FORCE_TILE=128x128), also when accumulating into C."""
+    the fused kernel (forced with sthip_debug_force_tile), also when accumulating into C."""
     M, N, K = shape
     A, B = _ints((M, K), 61), _ints((K, N), 62)
     Ag, Bg = _layout(A, ta), _layout(B, tb)
@@ -302,7 +296,7 @@ def test_fp32_batched_products(hip, monkeypatch, ta, tb, shape):
     C0 = _gauss((M, N), 65, 1.0, torch.float32).cuda()
     got = hip.gemm(Ag, Bg, algo="strassen", levels=1)
     acc = hip.gemm(Ag, Bg, out=C0.clone(), algo="strassen", levels=1, accumulate=True)
-    monkeypatch.setenv("STHIP_FORCE_TILE", "128x128")
+    force_tile("128x128")
     fused = hip.gemm(Ag, Bg, algo="strassen", levels=1)
     ref = Ag.double() @ Bg.double()
     rel = lambda X, R: float(torch.linalg.norm(X.double() - R) / torch.linalg.norm(R))
@@ -366,11 +360,11 @@ def test_autograd_matmul(hip):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
 @pytest.mark.parametrize("tb", [False, True])
-def test_every_pipelined_tile_exact(hip, monkeypatch, tile, dtype, algo, tb):
+def test_every_pipelined_tile_exact(hip, force_tile, tile, dtype, algo, tb):
     """The tile table picks by size; force each pipelined kernel on a small aligned problem so
     that all of them are checked bit for bit (integer inputs), with two batch entries, and again
     in accumulate mode with an fp32 result."""
-    monkeypatch.setenv("STHIP_FORCE_TILE", tile)
+    force_tile(tile)
     b, M, N, K = 2, 1024, 1024, 512
     A, B = _ints((b, M, K), 51, -1, 1, dtype), _ints((b, K, N), 52, -1, 1, dtype)
     want = A.double() @ B.double()
@@ -394,12 +388,12 @@ def test_every_pipelined_tile_exact(hip, monkeypatch, tile, dtype, algo, tb):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("pad,off", [(0, 0), (8, 0), (4, 0), (8, 4)])
 @pytest.mark.parametrize("algo,levels", [("classic", 0), ("strassen", 1)])
-def test_large_tile_store_alignment(hip, monkeypatch, dtype, pad, off, algo, levels):
+def test_large_tile_store_alignment(hip, force_tile, dtype, pad, off, algo, levels):
     """The 256 x 256 kernel stores 16-bit results sixteen bytes per lane when C, its rows and its
     strides are 16-byte aligned, eight bytes per lane otherwise: results written into a view of a
     wider buffer (row stride N + pad, first column off) are exact either way and the columns
     outside the view stay untouched."""
-    monkeypatch.setenv("STHIP_FORCE_TILE", "256x256")
+    force_tile("256x256")
     M, N, K = 1024, 512, 128
     A, B = _ints((M, K), 61, -1, 1, dtype), _ints((K, N), 62, -1, 1, dtype)   # |C| <= 128: exact in 16 bit
     want = A.double() @ B.double()
@@ -448,22 +442,22 @@ def test_fp32_large_tile_gaussian(hip):
 
 
 @pytest.mark.parametrize("tb", [False, True])
-def test_fp32_two_levels_fused_passes_bit_identical(hip, tb):
-    """Two fp32 levels on the 49-product form: the one-pass sums and the one-pass recombination
-    add in the same order as the separate passes (stage-mask bits 4 and 5 off), so the results
-    are the same bits, and both are inside the fp32 tolerance against fp64."""
+def test_fp32_two_levels_flat_against_host_recursion(hip, tb):
+    """Two fp32 levels as sums / 49 grouped products / one recombination pass against the host
+    recursion (stage-mask bit 3 off): nothing is rounded in either, so they differ by summation
+    order only, and both are inside the fp32 tolerance against fp64."""
     from strassen_hip import _capi
     M, N, K = 4096, 4096, 512
     A, B = _gauss((M, K), 91, 1.0, torch.float32), _gauss((K, N), 92, 1.0, torch.float32)
     Ag, Bg = A.cuda(), _layout(B, tb)
     fused = hip.gemm(Ag, Bg, algo="strassen", levels=2)
     lib = _capi.load()
-    prev = lib.sthip_debug_set_stages(15)
+    prev = lib.sthip_debug_set_stages(7)
     try:
-        separate = hip.gemm(Ag, Bg, algo="strassen", levels=2)
+        recursive = hip.gemm(Ag, Bg, algo="strassen", levels=2)
     finally:
         lib.sthip_debug_set_stages(prev)
-    assert torch.equal(fused, separate)
+    assert float(torch.linalg.norm(fused.double() - recursive.double()) / torch.linalg.norm(fused.double())) <= TOL[torch.float32]
     want = A.double() @ B.double()
     err = float(torch.linalg.norm(fused.cpu().double() - want) / torch.linalg.norm(want))
     assert err <= TOL[torch.float32]

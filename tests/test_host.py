@@ -12,9 +12,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _header_symbols():
-    text = open(os.path.join(ROOT, "include", "strassen_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(sthip_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in ("strassen_hip.h", "strassen_hip_debug.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(sthip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -23,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     names = _header_symbols()
     assert len(names) >= 8
     for n in names:
-        assert hasattr(lib, n), f"{n} declared in include/strassen_hip.h but not exported"
+        assert hasattr(lib, n), f"{n} declared in include/ but not exported"
         assert n in _capi.SIGNATURES, f"{n} has no ctypes prototype"
     assert set(_capi.SIGNATURES) == set(names)
     assert lib.sthip_version() == 100
@@ -80,15 +83,17 @@ def test_argument_errors_need_no_gpu():
     assert lib.sthip_workspace_bytes(1, 1000, 1024, 1024, 2, 2, 1, 1) == 0
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 0, 1) == 0
     # Two levels: five S_A, five S_B and seven fp32 M buffers of half size, plus the leaf's workspace
-    # (host recursion), or -- for tile-aligned 16-bit problems, which may run as one 49-product launch --
-    # ten half-size sums, 70 quarter-size sums, 49 quarter-size products and seven half-size products;
-    # the query covers whichever is larger.
+    # (host recursion; a leaf under an upper level hands its result over in fp32 and keeps its seven
+    # products in fp32 too), or -- for tile-aligned 16-bit problems, which may run as one 49-product
+    # launch -- ten half-size sums, 70 quarter-size sums and 49 quarter-size products; the query covers
+    # whichever is larger.
     upper = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
-    flat = lambda h: 10 * h * h * 2 + (70 + 49) * (h // 2) ** 2 * 2 + 7 * h * h * 2
+    inner_sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
+    flat = lambda h: 10 * h * h * 2 + (70 + 49) * (h // 2) ** 2 * 2
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
-    assert two == max(upper(512) + sums(256), flat(512))
+    assert two == max(upper(512) + inner_sums(256), flat(512))
     three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
-    assert three == upper(512) + max(upper(256) + sums(128), flat(256))
+    assert three == upper(512) + max(upper(256) + inner_sums(128), flat(256))
     # fp32 never takes the one-launch form
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4 + f32(256)
 
