@@ -10,11 +10,23 @@ line:
   value / ms_per_step   effective TFLOP/s = 2MNK / t (the classical flop count, as the
                         reference's main_profiling.py:190,216-217 counts it) over exactly K
                         back-to-back steps between two synchronisations
-  hipblaslt_*           torch.matmul (hipBLASLt) on the same tensors, same protocol, and the ratio
+  step_ms               min / median / mean over K further steps timed one by one with HIP events
+  flushed_ms            median over steps that each follow a write of a 512 MiB buffer (larger than
+                        the 256 MiB memory-side cache), the protocol of the reference's do_bench
+                        (main_profiling.py:197); flushed_ratio_vs_hipblaslt is the same for both sides
+  hipblaslt_*           torch.matmul (hipBLASLt) on the same tensors, same protocols, and the ratios
   roofline              the dominant kernel (the grouped-GEMM launch) timed alone with HIP events
-                        on the stream it runs on, against the MI355X dense MFMA peak
+                        on the stream it runs on, against the MI355X dense MFMA peak.  frac divides
+                        the classical flop count of the call by that kernel's time (the convention
+                        of the metric); frac_executed counts only the matrix work the kernel
+                        executes (7/8 per level); frac_whole_call divides by the whole call's time.
+                        traffic is not measured in this run: traffic_source names the committed
+                        rocprofv3 counter summary it is read from.
   cpu_baseline          the CPU oracle (a restatement of the reference's torch recursion) on the
                         host cores, best of 3
+
+The clocks of the card ramp for the first 20-30 ms of matrix work in a fresh process (both this
+library and hipBLASLt run 10-15 % slower there), so the default warm-up is 50 steps.
 
 `--workload copy_1gib` runs a plain 1 GiB device copy instead; it exists to calibrate the
 FETCH_SIZE / WRITE_SIZE counters when the HBM traffic of the kernels is measured with rocprofv3.
@@ -85,6 +97,21 @@ def time_gpu(fn, steps, warmup):
     return wall, start.elapsed_time(stop) * 1e-3
 
 
+def time_steps(fn, steps, flush=None):
+    """Every step timed on its own with a pair of HIP events; with `flush`, a write of that buffer
+    (larger than the memory-side cache) goes before every step, outside its timed region."""
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in events:
+        if flush is not None:
+            flush.zero_()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in events)
+    return {"min": round(t[0], 4), "median": round(t[len(t) // 2], 4), "mean": round(sum(t) / len(t), 4)}
+
+
 def cpu_baseline(A, B, levels, dtype, algo):
     """The oracle (a restatement of the reference's torch recursion) on the host cores."""
     from oracle import strassen_oracle as O
@@ -129,12 +156,12 @@ def cpu_baseline(A, B, levels, dtype, algo):
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
     WRITE_SIZE and recorded in profiles/ (None if no such summary is committed)."""
-    path = os.path.join(ROOT, "profiles", f"gemm_kernel_{workload}_hbm_traffic.txt")
+    rel = os.path.join("profiles", f"gemm_kernel_{workload}_hbm_traffic.txt")
     try:
-        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
-        return float(m.group(1)) if m else None
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(os.path.join(ROOT, rel)).read(), re.M)
+        return (float(m.group(1)), rel) if m else (None, None)
     except OSError:
-        return None
+        return None, None
 
 
 def copy_calibration(steps):
@@ -151,8 +178,8 @@ def copy_calibration(steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="strassen1_8192_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--force-tile", default=None, choices=["128x128", "128x128g", "256x128", "256x256"],
@@ -203,8 +230,16 @@ def main():
         fn()   # leave `out` holding a complete result for the error figures below
 
     ref_out = torch.empty_like(out)
-    wall_b, ev_b = time_gpu(lambda: torch.matmul(Ag, Bg, out=ref_out), args.steps, args.warmup)
+    blas = lambda: torch.matmul(Ag, Bg, out=ref_out)
+    wall_b, ev_b = time_gpu(blas, args.steps, args.warmup)
     blas_tflops = flops * args.steps / wall_b / 1e12
+
+    # step by step, back to back and with the caches flushed before every step
+    stat_steps = min(args.steps, 100)
+    step_ms, blas_step_ms = time_steps(fn, stat_steps), time_steps(blas, stat_steps)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+    flushed, blas_flushed = time_steps(fn, stat_steps, flush), time_steps(blas, stat_steps, flush)
+    del flush
 
     # numerical error of the timed result against fp64 and against hipBLASLt's result
     exact = torch.matmul(Ag[0].double() if batch > 1 else Ag.double(), Bg[0].double() if batch > 1 else Bg.double())
@@ -216,8 +251,12 @@ def main():
     peak = PEAK_TFLOPS[DT_NAME[dtype]]
     achieved = flops / kernel_s / 1e12
     executed = (7.0 / 8.0) ** (levels if algo != "classic" else 0)
+    traffic, traffic_source = measured_traffic(args.workload)
+    metric = "effective TFLOP/s (2MNK/t) at 8192\u00b2 bf16; ratio vs hipBLASLt GEMM"
+    if args.workload != "strassen1_8192_bf16":
+        metric = f"effective TFLOP/s (2MNK/t) on {args.workload}; ratio vs hipBLASLt GEMM"
     result = {
-        "metric": "effective TFLOP/s (2MNK/t) at 8192\u00b2 bf16; ratio vs hipBLASLt GEMM",
+        "metric": metric,
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": DT_NAME[dtype], "data": "synthetic",
@@ -226,10 +265,16 @@ def main():
                    "workspace_bytes": nbytes, "force_tile": args.force_tile},
         "hipblaslt_tflops": round(blas_tflops, 2), "ratio_vs_hipblaslt": round(tflops / blas_tflops, 4),
         "hipblaslt_ms": round(wall_b / args.steps * 1e3, 4),
+        "step_ms": step_ms, "hipblaslt_step_ms": blas_step_ms,
+        "flushed_ms": flushed["median"], "hipblaslt_flushed_ms": blas_flushed["median"],
+        "flushed_ratio_vs_hipblaslt": round(blas_flushed["median"] / flushed["median"], 4),
         "mfma_peak_frac": round(tflops / peak, 4),
         "rel_fro_err_vs_fp64": err64, "hipblaslt_rel_fro_err_vs_fp64": err_blas,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload),
+                     "frac": round(achieved / peak, 4),
+                     "frac_executed": round(achieved * executed / peak, 4),
+                     "frac_whole_call": round(tflops / peak, 4),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "grouped GEMM launch of the call (stage mask 2)" if staged else "whole call",
                      "kernel_ms": round(kernel_s * 1e3, 4), "prepass_ms": round(prepass_s * 1e3, 4),
                      "recombine_ms": round(recombine_s * 1e3, 4),

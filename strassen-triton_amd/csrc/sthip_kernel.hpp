@@ -74,6 +74,16 @@ struct TileGeom {
 };
 
 // ------------------------------------------------------------------ element arithmetic
+// A load / store with a streaming (nontemporal) hint when `streaming` is set: data that is touched once
+// and is larger than the caches should not push the operand panels out of them; data that the next kernel
+// of the same call reads again and that fits should stay.
+template <class V> __device__ __forceinline__ V load_hinted(const V* p, int streaming) {
+    return streaming ? __builtin_nontemporal_load(p) : *p;
+}
+template <class V> __device__ __forceinline__ void store_hinted(V v, V* p, int streaming) {
+    if (streaming) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 // Taking the argument by value matters: __builtin_bit_cast applied directly to a vector

@@ -48,6 +48,7 @@ struct Gemm2Params {
     int tiles_m, tiles_n;
     int out_f32, accumulate, group_m;
     int c_wide;           // 256 x 256 kernel: C, its rows and its product / batch strides are 16-byte aligned
+    int c_stream;         // 256 x 256 kernel: store the result tiles with the streaming hint
 };
 
 __device__ __forceinline__ void wait_vmcnt(int n) {

@@ -309,7 +309,7 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
                 f32x4* d = reinterpret_cast<f32x4*>(dst);
                 f32x4 o = {v[0], v[1], v[2], v[3]};
                 if (P.accumulate) { o += *d; *d = o; }
-                else __builtin_nontemporal_store(o, d);
+                else store_hinted(o, d, P.c_stream);
             } else {
                 u32x2* d = reinterpret_cast<u32x2*>(dst);
                 if (P.accumulate) {
@@ -366,10 +366,11 @@ __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Para
     for (int r = 0; r < 16; ++r) {
         const int rr = ((8 * r + r8) >> 1) & 7;
         const u32x4 v = *reinterpret_cast<const u32x4*>(w + (8 * r + r8) * 128 + ((c16 ^ rr) * 16));
-        // streaming store: the tile is not read again by this launch, and a round of tiles is as
-        // large as the L2s, which hold the operand panels the neighbours are re-reading
-        // (measured: -1 % at 8192^3, -3 % at 16384^2 x 4096)
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + r * step));
+        // streaming store on large problems: the tile is not read again by this launch, and a round of
+        // tiles is as large as the L2s, which hold the operand panels the neighbours are re-reading
+        // (measured: -1 % at 8192^3, -3 % at 16384^2 x 4096); on problems whose products fit the
+        // memory-side cache the recombination pass finds them there with a plain store (-3 % at 4096^3)
+        store_hinted(v, reinterpret_cast<u32x4*>(dst + r * step), P.c_stream);
     }
 }
 
@@ -394,7 +395,7 @@ __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2
         for (int r = 0; r < 16; ++r) {
             const int rl = 4 * r + q;
             const f32x4 v = *reinterpret_cast<const f32x4*>(w + rl * 256 + ((l16 ^ (rl & 15)) * 16));
-            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + (int64_t)(64 * h + 4 * r) * P.c_rs));
+            store_hinted(v, reinterpret_cast<f32x4*>(dst + (int64_t)(64 * h + 4 * r) * P.c_rs), P.c_stream);
         }
     }
 }
