@@ -186,7 +186,7 @@ def strassen_matmul_n_layers(A: torch.Tensor, B: torch.Tensor, n_depth: int = 2,
     return _assemble(r(M1 + M4 - M5 + M7), r(M3 + M5), r(M2 + M4), r(M1 - M2 + M3 + M6))
 
 
-def strassen_matmul_two_layers(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+def strassen_matmul_two_layers(A: torch.Tensor, B: torch.Tensor, mm=torch.mm) -> torch.Tensor:
     """Fixed two-level recursion with the reference's validation (strassen.py:742-812).
 
     Raises ValueError with the reference's messages for non-square / n % 4 / n <= 0
@@ -199,7 +199,7 @@ def strassen_matmul_two_layers(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor
         raise ValueError("Matrix size must be divisible by 4 for two Strassen layers.")
     if not n > 0:
         raise ValueError("Matrix size must be positive.")
-    return strassen_matmul_n_layers(A, B, n_depth=2, fp32_agg=False)
+    return strassen_matmul_n_layers(A, B, n_depth=2, fp32_agg=False, mm=mm)
 
 
 # ---------------------------------------------------------------------------------------
@@ -375,7 +375,7 @@ def tile_kernel_semantics(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor,
 
 
 def linear_strassen_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
-                            depth: int = 1) -> torch.Tensor:
+                            depth: int = 1, mm=torch.mm) -> torch.Tensor:
     """model/layers.py:246-274: view to (M, D), M > D -> ValueError (:255-259), zero-pad
     rows to D (:261-262), Strassen product with weight.T (:264), slice, view, + bias."""
     *batch_dims, D_in = x.shape
@@ -388,9 +388,9 @@ def linear_strassen_forward(x: torch.Tensor, weight: torch.Tensor, bias: torch.T
             f"You MUST use the method that pads BOTH input and weights to PxP.")
     Xp = torch.nn.functional.pad(x.reshape(Mrows, D), (0, 0, 0, D - Mrows))
     if depth == 2:
-        out = strassen_matmul_two_layers(Xp, weight.T)
+        out = strassen_matmul_two_layers(Xp, weight.T, mm)
     else:
-        out = strassen_base(Xp, weight.T)
+        out = strassen_base(Xp, weight.T, mm)
     out = out[:Mrows, :D].reshape(*batch_dims, D)
     return out + bias if bias is not None else out
 

@@ -82,6 +82,10 @@ class LinearStrassen(nn.Linear):
         self.cache_weight_sums = cache_weight_sums
         self.weight_sums = strassen_hip.WeightSums()
 
+    def _levels_for(self, D: int) -> int:
+        """Levels strassen_matmul_n_layers(X, W.T, n_depth=self.depth) takes (fixed_strassen.py:157)."""
+        return max(1, practical_levels(D, reference_levels(D, self.depth)))
+
     def forward(self, input: Tensor):
         *batch_dims, D_in = input.shape
         assert D_in == self.in_features, "Input dim mismatch"
@@ -91,7 +95,7 @@ class LinearStrassen(nn.Linear):
             raise ValueError(
                 f"Input M ({M}) > D ({D}). Cannot pad input to DxD. "
                 f"You MUST use the method that pads BOTH input and weights to PxP.")
-        levels = max(1, practical_levels(D, reference_levels(D, self.depth)))
+        levels = self._levels_for(D)
         sums = self.weight_sums.get(self.weight, levels) if self.cache_weight_sums and M == D else None
         out = _LinearFn.apply(input.reshape(M, D), self.weight, self.bias, levels, sums)
         return out.view(*batch_dims, D)

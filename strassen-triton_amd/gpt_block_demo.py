@@ -6,8 +6,8 @@ projections), LayerNorm, feed-forward with 4 x expansion and SiLU, residuals.
     python gpt_block_demo.py [--dim 4096] [--heads 32] [--tokens 8192] [--dtype bf16] [--backward]
 
 The block runs eagerly; attention itself is torch's scaled_dot_product_attention in both runs,
-only the four Linear layers change (replace_linear_with_strassen(..., square_only=False): the
-square projection becomes LinearStrassen, the non-square ones LinearStrassenRect).
+only the four Linear layers change (replace_linear_with_strassen(..., square_only=False): all four
+become LinearStrassenRect, which takes any number of token rows).
 """
 from __future__ import annotations
 
@@ -55,6 +55,43 @@ def _time(fn, warmup: int = 3, runs: int = 10) -> float:
     return start.elapsed_time(stop) / runs
 
 
+def compare_block(dim: int, heads: int, tokens: int, dtype=torch.bfloat16, backward: bool = False,
+                  cache_weight_sums: bool = False, warmup: int = 3, runs: int = 10, verbose: bool = True) -> dict:
+    """Builds one block, swaps the Linear layers of a copy, and returns the times of both and the
+    relative difference of their outputs (and, with backward, of the input gradients)."""
+    torch.manual_seed(0)
+    std = Block(dim, heads, dtype=dtype)
+    ours = copy.deepcopy(std)
+    if verbose:
+        replace_linear_with_strassen(ours, min_size=128, depth=1, square_only=False, cache_weight_sums=cache_weight_sums)
+    else:
+        import contextlib, io
+        with contextlib.redirect_stdout(io.StringIO()):
+            replace_linear_with_strassen(ours, min_size=128, depth=1, square_only=False, cache_weight_sums=cache_weight_sums)
+    seq = min(1024, tokens)
+    x = torch.randn(tokens // seq, seq, dim, device="cuda", dtype=dtype)
+
+    def step(block):
+        if not backward:
+            with torch.no_grad():
+                return block(x)
+        block.zero_grad(set_to_none=True)
+        y = block(x)
+        y.float().square().mean().backward()
+        return y
+
+    rel = lambda got, ref: float(torch.linalg.norm(got.float() - ref.float()) / torch.linalg.norm(ref.float()))
+    with torch.no_grad():
+        res = {"dim": dim, "heads": heads, "tokens": tokens, "backward": backward, "rel_diff": rel(ours(x), std(x))}
+    if backward:
+        step(std), step(ours)
+        res["rel_diff_weight_grad"] = max(rel(po.grad, ps.grad) for (_, po), (_, ps) in
+                                          zip(ours.named_parameters(), std.named_parameters()) if ps.dim() == 2)
+    res["std_ms"], res["strassen_ms"] = _time(lambda: step(std), warmup, runs), _time(lambda: step(ours), warmup, runs)
+    res["replaced"] = sorted(type(m).__name__ for m in ours.modules() if type(m).__name__.startswith("LinearStrassen"))
+    return res
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--dim", type=int, default=4096)
@@ -67,32 +104,12 @@ def main() -> None:
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: this demo needs an MI355X")
-    dtype = _DTYPES[args.dtype]
-    torch.manual_seed(0)
-    std = Block(args.dim, args.heads, dtype=dtype)
-    ours = copy.deepcopy(std)
-    replace_linear_with_strassen(ours, min_size=128, depth=1, square_only=False,
-                                 cache_weight_sums=args.cache_weight_sums)
-    seq = min(1024, args.tokens)
-    x = torch.randn(args.tokens // seq, seq, args.dim, device="cuda", dtype=dtype)
-
-    def step(block):
-        if not args.backward:
-            with torch.no_grad():
-                return block(x)
-        block.zero_grad(set_to_none=True)
-        y = block(x)
-        y.float().square().mean().backward()
-        return y
-
-    with torch.no_grad():
-        ref, got = std(x).float(), ours(x).float()
-    rel = float(torch.linalg.norm(got - ref) / torch.linalg.norm(ref))
-    t_std, t_ours = _time(lambda: step(std)), _time(lambda: step(ours))
+    r = compare_block(args.dim, args.heads, args.tokens, _DTYPES[args.dtype], args.backward, args.cache_weight_sums)
     what = "forward + backward" if args.backward else "forward"
     print(f"block dim {args.dim}, {args.tokens} tokens, {args.dtype}, {what}:")
-    print(f"  nn.Linear       {t_std:9.3f} ms")
-    print(f"  Strassen layers {t_ours:9.3f} ms   ({t_std / t_ours:.2f}x)   output rel. difference {rel:.2e}")
+    print(f"  nn.Linear       {r['std_ms']:9.3f} ms")
+    print(f"  Strassen layers {r['strassen_ms']:9.3f} ms   ({r['std_ms'] / r['strassen_ms']:.2f}x)   "
+          f"output rel. difference {r['rel_diff']:.2e}")
 
 
 if __name__ == "__main__":

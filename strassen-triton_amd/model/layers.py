@@ -14,13 +14,20 @@ from strassen import _strassen_base, strassen_matmul_two_layers
 
 
 class LinearStrassen(_LinearStrassen):
-    """Same module as fixed_strassen.LinearStrassen with the constructor of reference
-    model/layers.py:232-244 (dtype defaults to None; depth 2 selects the two-layer product)."""
+    """Same module as fixed_strassen.LinearStrassen with the constructor and the depth rule of
+    reference model/layers.py:232-244: dtype defaults to None; depth 2 selects the two-layer
+    product, every other depth the one-level routine (there depth 3 is one level, not three).
+    strassen_func names the function of the reference-shaped surface that computes the same
+    product; forward itself goes through the fused Linear entry of the C ABI (no padding copy)."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype=None,
                  depth: int = 1, device: str = "cuda", cache_weight_sums: bool = False) -> None:
         super().__init__(in_features, out_features, bias, dtype, depth, device, cache_weight_sums)
         self.strassen_func = strassen_matmul_two_layers if depth == 2 else _strassen_base
+
+    def _levels_for(self, D: int) -> int:
+        from _levels import practical_levels
+        return max(1, practical_levels(D, 2 if self.depth == 2 else 1))
 
 
 class _RectLinearFn(torch.autograd.Function):
@@ -85,6 +92,7 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
                                                dtype=child.weight.dtype, depth=depth,
                                            cache_weight_sums=cache_weight_sums)
                 new_layer.weight.data.copy_(child.weight.data)
+                new_layer.weight_sums.clear()   # a write through .data does not move the version counter
                 if child.bias is not None:
                     new_layer.bias.data.copy_(child.bias.data)
                 setattr(module, name, new_layer)
@@ -95,6 +103,7 @@ def replace_linear_with_strassen(module: nn.Module, min_size: int = 128, depth: 
                                            dtype=child.weight.dtype, depth=depth,
                                            cache_weight_sums=cache_weight_sums)
                 new_layer.weight.data.copy_(child.weight.data)
+                new_layer.weight_sums.clear()   # a write through .data does not move the version counter
                 if child.bias is not None:
                     new_layer.bias.data.copy_(child.bias.data)
                 setattr(module, name, new_layer)

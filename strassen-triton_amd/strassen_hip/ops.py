@@ -231,13 +231,21 @@ def prepare_weight(weight: torch.Tensor, levels: int) -> torch.Tensor | None:
 
 class WeightSums:
     """Keeps the prepared sums of one weight tensor and forms them again when the tensor is
-    written (its version counter moves), replaced, or asked for at another depth."""
+    written (its version counter moves), replaced, or asked for at another depth.  A write through
+    `.data` does not move the counter: call clear() (or refresh()) after one."""
 
     def __init__(self) -> None:
         self.clear()
 
     def get(self, weight: torch.Tensor, levels: int) -> torch.Tensor | None:
-        key = (weight.data_ptr(), weight._version, tuple(weight.shape), weight.dtype, levels)
+        try:
+            version = weight._version
+        except RuntimeError:
+            # inference tensors (created under torch.inference_mode) track no version: nothing to key
+            # the kept sums on, so form them for this call only
+            self.clear()
+            return prepare_weight(weight, levels)
+        key = (weight.data_ptr(), version, tuple(weight.shape), weight.dtype, levels)
         same_tensor = self._owner is not None and self._owner() is weight
         if not same_tensor or key != self._key:
             self._sums = prepare_weight(weight, levels)
@@ -246,6 +254,8 @@ class WeightSums:
 
     def clear(self) -> None:
         self._key, self._sums, self._owner = None, None, None
+
+    refresh = clear
 
     # a copied or unpickled layer starts without sums and forms its own on first use
     def __getstate__(self):
