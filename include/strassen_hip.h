@@ -141,11 +141,23 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
  * row-major, all tensors contiguous; bias as in sthip_linear_strassen_forward.  The reference's
  * layer is square, a power of two and pads its input to D x D (model/layers.py:240, :255-262);
  * this is the same forward with those constraints lifted (no padding: sizes that are not tile
- * multiples take the kernels' edge tiles).  levels = 0 runs the classical product.
+ * multiples take the kernels' edge tiles).  levels = 0 runs the classical product; levels < 0 runs
+ * sthip_auto_levels(rows, out_features, in_features, dtype, -levels) levels, so that the layer never
+ * takes a Strassen path that is slower than the library's classical kernel on that shape.
  * Workspace as sthip_workspace_bytes(1, rows, out, in, dtype, dtype, STHIP_STRASSEN, levels). */
 int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y,
                          int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* How many Strassen levels (0 = the classical product, at most max_levels) make C = A x B of this
+ * shape fastest on MI355X, from measurements of this library's own kernels against each other
+ * (sweep of M, N, K in 768 .. 16384, both layouts of B): one level pays where the classical product
+ * cannot fill the chip but the seven half-size products side by side can (at most 128 output tiles
+ * of 128 x 128 and k >= 4096: weight gradients), and from about 16384^3 up (fp32: 8192^3); a second
+ * level from 32768^3 (fp32: 16384^3), a third from 65536^3 (fp32: 32768^3).  sthip_linear_forward
+ * applies this rule when its `levels` argument is negative.  No counterpart in the reference, whose
+ * only cutoff is the min_size of replace_linear_with_strassen (model/layers.py:279-300). */
+int sthip_auto_levels(int64_t M, int64_t N, int64_t K, int dtype, int max_levels);
 
 /* A Linear layer whose weight stays put between calls (inference, or the reference's benchmark
  * main_profiling.py:94-245, which times repeated forwards of one layer): the quadrant sums of

@@ -1629,9 +1629,25 @@ static int finish_bias(Call& cx, const void* bias, void* y, int64_t rows, int64_
     return check_launch("add_bias");
 }
 
+// Levels that make this shape fastest (see sthip_auto_levels in the header for the measurements).
+static int auto_levels(int64_t M, int64_t N, int64_t K, int dt, int max_levels) {
+    if (max_levels <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t smallest = std::min(M, std::min(N, K));
+    const int64_t big1 = dt == STHIP_F32 ? 8192 : 16384;   // every extent at least this: one level pays
+    int levels = 0;
+    if (smallest >= big1 || (smallest >= big1 / 2 && K >= big1 && M * N >= big1 * big1 / 2)) levels = 1;
+    if (smallest >= 2 * big1) levels = 2;
+    if (smallest >= 4 * big1) levels = 3;
+    // few output tiles, long k: one classical product leaves most CUs idle, seven half-size ones do not
+    if (levels == 0 && dt != STHIP_F32 && ceil_div(M, 128) * ceil_div(N, 128) <= 128 && K >= 4096 &&
+        M % 256 == 0 && N % 256 == 0 && K % 128 == 0) levels = 1;
+    return std::min(levels, max_levels);
+}
+
 static int linear_forward_impl(Call& cx, const void* x, const void* W, const void* bias, void* y,
                                int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                                void* workspace, size_t workspace_bytes) {
+    if (levels < 0) levels = auto_levels(rows, out_features, in_features, dtype, std::min(-levels, 8));
     int rc = check_common(x, W, y, 1, rows, out_features, in_features, dtype, dtype, STHIP_STRASSEN, levels);
     if (rc) return rc;
     if (rows == 0 || out_features == 0) return STHIP_OK;
@@ -1776,6 +1792,10 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
                          void* workspace, size_t workspace_bytes, void* stream) {
     Call cx = begin_call(stream);
     return linear_forward_impl(cx, x, W, bias, y, rows, in_features, out_features, dtype, levels, workspace, workspace_bytes);
+}
+
+int sthip_auto_levels(int64_t M, int64_t N, int64_t K, int dtype, int max_levels) {
+    return auto_levels(M, N, K, dtype, max_levels);
 }
 
 size_t sthip_linear_weight_sums_bytes(int64_t in_features, int64_t out_features, int dtype, int levels) {

@@ -131,12 +131,14 @@ _GPT2_LINEARS = [("qkv", 768, 2304), ("attn_proj", 768, 768), ("mlp_up", 768, 30
 @torch.no_grad()
 def profile_gpt2_linears(tokens: int = 8192, dtype=torch.bfloat16) -> list[dict]:
     """Forward x W^T, dgrad dY W and wgrad dY^T X of each GPT-2-small Linear for `tokens`
-    rows, one Strassen level on strided views against torch.matmul on the same views."""
+    rows on strided views: torch.matmul, one Strassen level, the library's classical kernel, and
+    what the measured cutoff picks between the latter two (levels = -1, the default of
+    LinearStrassenRect)."""
     import strassen_hip
     flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
     rows = []
     print(f"{'layer':>10s} | {'pass':>5s} | {'M x N x K':>18s} | {'matmul ms':>10s} | {'strassen ms':>11s} | "
-          f"{'classic ms':>10s} | {'matmul TF':>9s} | {'strassen TF':>11s} | {'rel err':>9s}")
+          f"{'classic ms':>10s} | {'cutoff ms':>9s} | {'levels':>6s} | {'matmul TF':>9s} | {'strassen TF':>11s} | {'rel err':>9s}")
     for name, d_in, d_out in _GPT2_LINEARS:
         x = torch.randn(tokens, d_in, device="cuda", dtype=dtype) * 0.02
         w = torch.randn(d_out, d_in, device="cuda", dtype=dtype) * 0.02
@@ -150,13 +152,16 @@ def profile_gpt2_linears(tokens: int = 8192, dtype=torch.bfloat16) -> list[dict]
             t_str = _bench(lambda: strassen_hip.gemm(a, b, out, workspace=ws), 10, 50, flush)
             err = float(torch.linalg.norm(out.double() - ref) / torch.linalg.norm(ref))
             t_cls = _bench(lambda: strassen_hip.gemm(a, b, out, algo="classic", levels=0), 10, 50, flush)
+            t_auto = _bench(lambda: strassen_hip.gemm(a, b, out, levels=-1, workspace=ws), 10, 50, flush)
+            picked = strassen_hip.auto_levels(M, N, K, dtype, 1)
             tf = lambda t: 2.0 * M * N * K / (min(t) * 1e-3) / 1e12
             r = dict(layer=name, which=which, M=M, N=N, K=K, std_ms=min(t_std), strassen_ms=min(t_str),
-                     classic_ms=min(t_cls), std_tflops=tf(t_std), strassen_tflops=tf(t_str), rel_err=err)
+                     classic_ms=min(t_cls), cutoff_ms=min(t_auto), cutoff_levels=picked,
+                     std_tflops=tf(t_std), strassen_tflops=tf(t_str), rel_err=err)
             rows.append(r)
             print(f"{name:>10s} | {which:>5s} | {f'{M}x{N}x{K}':>18s} | {r['std_ms']:>10.4f} | {r['strassen_ms']:>11.4f} | "
-                  f"{r['classic_ms']:>10.4f} | {r['std_tflops']:>9.1f} | {r['strassen_tflops']:>11.1f} | {err:>9.2e}",
-                  flush=True)
+                  f"{r['classic_ms']:>10.4f} | {r['cutoff_ms']:>9.4f} | {picked:>6d} | {r['std_tflops']:>9.1f} | "
+                  f"{r['strassen_tflops']:>11.1f} | {err:>9.2e}", flush=True)
     return rows
 
 

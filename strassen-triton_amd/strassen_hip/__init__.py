@@ -1,7 +1,8 @@
 """Host side of the MI355X Strassen library: tensors in, C-ABI calls out."""
-from .ops import (ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD, StrassenMatmul, WeightSums, gemm, linear_forward,
+from . import _capi
+from .ops import (ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD, StrassenMatmul, WeightSums, auto_levels, gemm, linear_forward,
                   linear_forward_any, matmul, prepare_weight, run_accumulate, workspace_bytes)
 
 __all__ = ["gemm", "matmul", "run_accumulate", "linear_forward", "linear_forward_any", "StrassenMatmul", "workspace_bytes",
-           "prepare_weight", "WeightSums",
+           "prepare_weight", "WeightSums", "auto_levels",
            "ALGO_CLASSIC", "ALGO_STRASSEN", "ALGO_WINOGRAD"]

@@ -27,6 +27,7 @@ SIGNATURES = {
                                     _vp, _sz, _vp]),
     "sthip_linear_strassen_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp, _sz, _vp]),
     "sthip_linear_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),
+    "sthip_auto_levels": (_int, [_i64, _i64, _i64, _int, _int]),
     "sthip_linear_weight_sums_bytes": (_sz, [_i64, _i64, _int, _int]),
     "sthip_linear_prepare_weight": (_int, [_vp, _i64, _i64, _int, _int, _vp, _sz, _vp]),
     "sthip_linear_forward_prepared": (_int, [_vp, _vp, _vp, _sz, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp, _sz, _vp]),

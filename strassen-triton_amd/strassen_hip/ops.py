@@ -69,13 +69,24 @@ def workspace_bytes(A: torch.Tensor, B: torch.Tensor, *, algo="strassen", levels
                                               _dtype_code(out_dtype or A.dtype), algo, levels)
 
 
+def auto_levels(M: int, N: int, K: int, dtype: torch.dtype, max_levels: int = 1) -> int:
+    """Levels (0 = classical, at most max_levels) the library's measured cutoff picks for an
+    M x K by K x N product (sthip_auto_levels)."""
+    return _capi.load().sthip_auto_levels(M, N, K, _dtype_code(dtype), max_levels)
+
+
 def gemm(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor | None = None, *, algo="strassen",
          levels: int = 1, accumulate: bool = False, out_dtype: torch.dtype | None = None,
          workspace: torch.Tensor | None = None) -> torch.Tensor:
-    """out (+)= A @ B through sthip_gemm.  A: (b,) M x K, B: (b,) K x N, same dtype."""
+    """out (+)= A @ B through sthip_gemm.  A: (b,) M x K, B: (b,) K x N, same dtype.
+    levels < 0: at most -levels levels, as many as the measured cutoff picks for the shape."""
     _require_gpu(A, B)
     lib = _capi.load()
     algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    if levels < 0:
+        levels = auto_levels(A.shape[-2], B.shape[-1], A.shape[-1], A.dtype, -levels)
+        if levels == 0:
+            algo = ALGO_CLASSIC
     if A.dim() != B.dim() or A.dim() not in (2, 3):
         raise ValueError(f"expected two 2-D or two 3-D tensors, got {tuple(A.shape)} and {tuple(B.shape)}")
     if A.dtype != B.dtype:
@@ -192,12 +203,14 @@ def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tens
         raise ValueError(f"shape mismatch: {tuple(x2d.shape)} @ {tuple(weight.shape)}^T")
     x2d, weight = x2d.contiguous(), weight.contiguous()
     dt = _dtype_code(x2d.dtype)
+    if levels < 0:
+        levels = lib.sthip_auto_levels(rows, d_out, d_in, dt, -levels)
     y = torch.empty((rows, d_out), dtype=x2d.dtype, device=x2d.device)
     nbytes = lib.sthip_workspace_bytes(1, rows, d_out, d_in, dt, dt, ALGO_STRASSEN, levels)
     ws, ws_ptr = _workspace(nbytes, x2d.device)
     b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
     with torch.cuda.device(x2d.device):
-        if weight_sums is not None:
+        if weight_sums is not None and levels > 0:
             _capi.check(lib.sthip_linear_forward_prepared(x2d.data_ptr(), weight.data_ptr(), weight_sums.data_ptr(),
                                                           weight_sums.numel(), b_ptr, y.data_ptr(),
                                                           rows, d_in, d_out, dt, levels, ws_ptr, nbytes, _stream()))

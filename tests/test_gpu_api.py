@@ -126,7 +126,7 @@ def test_linear_strassen_rect_forward_backward(dtype, shape):
     rows, d_in, d_out = shape
     tol = 1e-5 if dtype == torch.float32 else 2e-2
     g = torch.Generator().manual_seed(7)
-    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda")
+    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda", cutoff=False)
     x = (torch.randn(rows, d_in, generator=g) * 0.5).to(dtype).cuda().requires_grad_()
     dy = (torch.randn(rows, d_out, generator=g) * 0.5).to(dtype).cuda()
     y = lin(x)
@@ -241,7 +241,7 @@ def test_linear_strassen_rect_bias_in_the_recombination_pass(dtype):
     from model.layers import LinearStrassenRect
     rows, d_in, d_out = 2048, 1024, 3072
     g = torch.Generator().manual_seed(33)
-    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda")
+    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda", cutoff=False)
     with torch.no_grad():
         lin.weight.copy_((torch.randn(d_out, d_in, generator=g) * d_in ** -0.5).to(dtype))
         lin.bias.copy_(torch.randn(d_out, generator=g).to(dtype))
@@ -305,8 +305,9 @@ def test_layers_keep_weight_sums_between_calls(depth):
     from model.layers import LinearStrassen, LinearStrassenRect
     g = torch.Generator().manual_seed(8 + depth)
     for make, rows, d_in, d_out in ((LinearStrassen, 2048, 2048, 2048), (LinearStrassenRect, 1024, 1024, 3072)):
-        plain = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda")
-        keep = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda", cache_weight_sums=True)
+        kw = {"cutoff": False} if make is LinearStrassenRect else {}
+        plain = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda", **kw)
+        keep = make(d_in, d_out, bias=True, dtype=torch.bfloat16, depth=depth, device="cuda", cache_weight_sums=True, **kw)
         with torch.no_grad():
             plain.weight.copy_((torch.randn(d_out, d_in, generator=g) * d_in ** -0.5).to(torch.bfloat16))
             plain.bias.copy_(torch.randn(d_out, generator=g).to(torch.bfloat16))

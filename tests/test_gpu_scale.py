@@ -91,14 +91,22 @@ def test_linear_strassen_4096_against_the_oracle(depth, rows):
     assert err64 <= TOL16 and err <= TOL16 * (1 if depth == 1 else 2) and err64 <= ora64 * 1.05
 
 
+@pytest.mark.parametrize("cutoff", [False, True])
 @pytest.mark.parametrize("d_in,d_out", [(768, 2304), (768, 768), (768, 3072), (3072, 768)])
-def test_gpt2_linear_shapes_through_the_autograd_layer(d_in, d_out):
+def test_gpt2_linear_shapes_through_the_autograd_layer(d_in, d_out, cutoff):
     """The GPT-2-small Linear shapes with 8192 token rows through LinearStrassenRect: forward,
     input gradient and weight gradient against the oracle's one-level product on the same
-    operands (strassen_general: fp32 aggregation, products in bf16)."""
+    operands (strassen_general: fp32 aggregation, products in bf16).  cutoff=False runs one
+    Strassen level in all three products; with the measured cutoff (the default) forward and
+    input gradient run the classical kernel on these shapes and the weight gradients of the
+    layers with at most 128 output tiles keep their level."""
+    import strassen_hip
     from model.layers import LinearStrassenRect
     rows, dtype = 8192, torch.bfloat16
-    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda")
+    if cutoff:
+        assert strassen_hip.auto_levels(rows, d_out, d_in, dtype, 1) == 0
+        assert strassen_hip.auto_levels(d_out, d_in, rows, dtype, 1) == (1 if d_in * d_out <= 128 * 128 * 128 else 0)
+    lin = LinearStrassenRect(d_in, d_out, bias=True, dtype=dtype, device="cuda", cutoff=cutoff)
     w, b = _gauss((d_out, d_in), 111, 0.02, dtype), _gauss((d_out,), 112, 0.02, dtype)
     with torch.no_grad():
         lin.weight.copy_(w)

@@ -177,3 +177,26 @@ def test_product_code_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_measured_cutoff_rule():
+    """sthip_auto_levels: host-only arithmetic.  Classical for the forward shapes of a small
+    transformer, one level for its weight gradients (few output tiles, long k) and for very large
+    products, more levels only beyond that; never more than max_levels."""
+    from strassen_hip import _capi
+    lib = _capi.load()
+    bf16, f32 = 2, 0
+    assert lib.sthip_auto_levels(8192, 2304, 768, bf16, 1) == 0
+    assert lib.sthip_auto_levels(8192, 8192, 8192, bf16, 2) == 0
+    assert lib.sthip_auto_levels(768, 768, 8192, bf16, 1) == 1
+    assert lib.sthip_auto_levels(2304, 768, 8192, bf16, 1) == 1
+    assert lib.sthip_auto_levels(3072, 768, 8192, bf16, 1) == 0        # 144 output tiles: the classical kernel fills enough CUs
+    assert lib.sthip_auto_levels(768, 768, 2048, bf16, 1) == 0         # k too short to pay for the passes
+    assert lib.sthip_auto_levels(16384, 16384, 16384, bf16, 3) == 1
+    assert lib.sthip_auto_levels(32768, 32768, 32768, bf16, 3) == 2
+    assert lib.sthip_auto_levels(32768, 32768, 32768, bf16, 1) == 1
+    assert lib.sthip_auto_levels(8192, 8192, 8192, f32, 3) == 1
+    assert lib.sthip_auto_levels(16384, 16384, 16384, f32, 3) == 2
+    assert lib.sthip_auto_levels(4096, 4096, 4096, f32, 3) == 0
+    assert lib.sthip_auto_levels(768, 768, 8192, f32, 1) == 0
+    assert lib.sthip_auto_levels(8192, 8192, 8192, bf16, 0) == 0 and lib.sthip_auto_levels(0, 8, 8, bf16, 1) == 0
