@@ -151,12 +151,14 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
 
 /* How many Strassen levels (0 = the classical product, at most max_levels) make C = A x B of this
  * shape fastest on MI355X, from measurements of this library's own kernels against each other
- * (sweep of M, N, K in 768 .. 16384, both layouts of B): one level pays where the classical product
- * cannot fill the chip but the seven half-size products side by side can (at most 128 output tiles
- * of 128 x 128 and k >= 4096: weight gradients), and from about 16384^3 up (fp32: 8192^3); a second
- * level from 32768^3 (fp32: 16384^3), a third from 65536^3 (fp32: 32768^3).  sthip_linear_forward
- * applies this rule when its `levels` argument is negative.  No counterpart in the reference, whose
- * only cutoff is the min_size of replace_linear_with_strassen (model/layers.py:279-300). */
+ * (sweep of M, N, K in 768 .. 16384, both layouts of B).  16-bit: one level where the classical
+ * product cannot fill the chip but the seven half-size products side by side can (at most 128
+ * output tiles of 128 x 128 and k >= 4096: weight gradients), and from about 16384^3 up; a second
+ * level from 32768^3, a third from 65536^3.  fp32: one level from 5e11 flop (8192 x 8192 x 4096), two
+ * from 1e12 (8192^3), three from 32768^3, and one level for products too small for the large-tile
+ * kernel.  sthip_linear_forward applies this rule when its `levels` argument is negative.  No
+ * counterpart in the reference, whose only cutoff is the min_size of replace_linear_with_strassen
+ * (model/layers.py:279-300). */
 int sthip_auto_levels(int64_t M, int64_t N, int64_t K, int dtype, int max_levels);
 
 /* A Linear layer whose weight stays put between calls (inference, or the reference's benchmark

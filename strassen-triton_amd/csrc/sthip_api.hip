@@ -1629,18 +1629,36 @@ static int finish_bias(Call& cx, const void* bias, void* y, int64_t rows, int64_
     return check_launch("add_bias");
 }
 
-// Levels that make this shape fastest (see sthip_auto_levels in the header for the measurements).
+// Levels that make this shape fastest, from a sweep of M, N, K over 768 .. 16384 (both layouts of
+// B) timing the classical kernel, one level and two levels of this library against each other.
 static int auto_levels(int64_t M, int64_t N, int64_t K, int dt, int max_levels) {
     if (max_levels <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
     const int64_t smallest = std::min(M, std::min(N, K));
-    const int64_t big1 = dt == STHIP_F32 ? 8192 : 16384;   // every extent at least this: one level pays
+    const double flops = 2.0 * (double)M * (double)N * (double)K;
+    const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
     int levels = 0;
-    if (smallest >= big1 || (smallest >= big1 / 2 && K >= big1 && M * N >= big1 * big1 / 2)) levels = 1;
-    if (smallest >= 2 * big1) levels = 2;
-    if (smallest >= 4 * big1) levels = 3;
-    // few output tiles, long k: one classical product leaves most CUs idle, seven half-size ones do not
-    if (levels == 0 && dt != STHIP_F32 && ceil_div(M, 128) * ceil_div(N, 128) <= 128 && K >= 4096 &&
-        M % 256 == 0 && N % 256 == 0 && K % 128 == 0) levels = 1;
+    if (dt == STHIP_F32) {
+        // the fp32 matrix cores are 16 x slower than the 16-bit ones while the passes only double:
+        // one level pays from 5e11 flop (8192 x 8192 x 4096: 1.05 x the classical kernel), a second
+        // from 1e12 (8192^3: 1.09 x, 16384^3: 1.23 x), a third from 32768^3 (1.32 x against 1.22 x)
+        if (std::min(M, N) >= 4096 && K >= 4096 && flops >= 5e11) levels = 1;
+        if (smallest >= 4096 && flops >= 1e12) levels = 2;
+        if (smallest >= 32768) levels = 3;
+        // fewer than 224 tiles of 256 x 256: the classical product runs on the 128 x 128 kernel, the
+        // seven half-size products of a level fill the large-tile kernel or run as one batch (1.3 - 1.8 x)
+        if (levels == 0 && tiles256 < 224 && M >= 1024 && N >= 1024 && K >= 1024 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0)
+            levels = 1;
+    } else {
+        // 16-bit: the passes of a level cost about 14 n^2 bytes against n^3 / 4 flop saved: break-even
+        // near 16384^3 (1.02 - 1.05 x there, 0.92 x at 8192^3); a second level from 32768^3, a third from 65536^3
+        if (smallest >= 16384 || (smallest >= 8192 && K >= 16384 && M * N >= (int64_t)8192 * 16384)) levels = 1;
+        if (smallest >= 32768) levels = 2;
+        if (smallest >= 65536) levels = 3;
+        // at most 128 output tiles of 128 x 128 and a long k (weight gradients): one classical product
+        // leaves most CUs idle, seven half-size ones side by side do not (1.1 - 1.5 x from k = 4096)
+        if (levels == 0 && ceil_div(M, 128) * ceil_div(N, 128) <= 128 && K >= 4096 &&
+            M % 256 == 0 && N % 256 == 0 && K % 128 == 0) levels = 1;
+    }
     return std::min(levels, max_levels);
 }
 
