@@ -17,7 +17,10 @@ int sthip_debug_transpose_read(void* out, void* stream);
 
 /* Selects which stages of the pipelined paths later calls run (bit 0 = quadrant-sum pre-pass,
  * bit 1 = grouped GEMM, bit 2 = recombination pass; bit 3 lets two-level calls run as one
- * 49-product launch instead of the host recursion; default 15) and returns the previous mask.
+ * 49-product launch instead of the host recursion; bit 4 runs large one-level 16-bit Strassen
+ * calls as ONE launch whose workgroups are the sums, the product tiles and the recombination --
+ * same bits, slower than the three launches on MI355X, hence off by default; default 15) and
+ * returns the previous mask.
  * With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so the
  * dominant kernel can be timed alone. */
 int sthip_debug_set_stages(int mask);

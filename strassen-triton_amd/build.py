@@ -43,6 +43,7 @@ def _units():
             units.append((f"sthip_inst3_{t}_{a}.o", "sthip_inst3.hip",
                           [f"-DSTHIP_INST_TYPE={t}", f"-DSTHIP_INST_ALGO={a}"]))
         units.append((f"sthip_inst4_{t}.o", "sthip_inst4.hip", [f"-DSTHIP_INST_TYPE={t}"]))
+        units.append((f"sthip_inst5_{t}.o", "sthip_inst5.hip", [f"-DSTHIP_INST_TYPE={t}"]))
     units.append(("sthip_inst4_0.o", "sthip_inst4.hip", ["-DSTHIP_INST_TYPE=0"]))
     return units
 

@@ -20,9 +20,11 @@ static thread_local char g_err[512] = "";
 // Process-wide debug switches (include/strassen_hip_debug.h).  Every public entry point reads them
 // once, into its Call; nothing below an entry point looks at them again.
 // Stages of the pipelined path that run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
-// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch.
-constexpr int kAllStages = 15;
-static std::atomic<int> g_debug_stages{kAllStages};
+// bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch, bit 4 = one level
+// may run as ONE launch (sums, products and recombination as work items of one grid).
+constexpr int kAllStages = 31;
+constexpr int kDefaultStages = 15;   // the one-launch form is slower than the three launches (sthip_kernel5.hpp): off unless asked for
+static std::atomic<int> g_debug_stages{kDefaultStages};
 // Forced tile: 0 = the tile table decides, 2 = 128 x 128, 3 = 256 x 128, 4 = 256 x 256, 5 = 128 x 128 with
 // the seven products as separate outputs; -1 = not set yet (the first call reads STHIP_FORCE_TILE).
 static std::atomic<int> g_debug_tile{-1};
@@ -75,6 +77,10 @@ static const LaunchTable3* table3_for(int dt, int algo) {
         case 6: return &kLaunch3_2_0; case 7: return &kLaunch3_2_1; case 8: return &kLaunch3_2_2;
     }
     return nullptr;
+}
+
+static const LaunchTable5* table5_for(int dt) {
+    return dt == STHIP_F16 ? &kLaunch5_1 : dt == STHIP_BF16 ? &kLaunch5_2 : nullptr;
 }
 
 static const LaunchTable3* table4_for(int dt) {
@@ -339,8 +345,12 @@ static const signed char kWinB[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0,
 // the 256 x 128 kernel parks one accumulator tile per workgroup (at most Mh x Nh floats).
 // (prod_es = 4: the seven products kept in fp32, for 16-bit operands with an fp32 result.)
 static size_t products_bytes(int64_t Mh, int64_t Nh, int prod_es = 2) { return 7 * align256(Mh * Nh * prod_es); }
-static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh, int prod_es = 2) {
+// (+ 256 bytes at the end: the dependency counters of the one-launch form)
+static size_t prepass_body_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh, int prod_es = 2) {
     return (size_t)batch * (5 * (align256(Mh * Kh * 2) + align256(Kh * Nh * 2)) + products_bytes(Mh, Nh, prod_es));
+}
+static size_t prepass_bytes(int64_t batch, int64_t Mh, int64_t Nh, int64_t Kh, int prod_es = 2) {
+    return prepass_body_bytes(batch, Mh, Nh, Kh, prod_es) + 256;
 }
 
 // Recombination of the seven 16-bit products of one level (kernel order: Strassen
@@ -379,7 +389,7 @@ struct PreparedSums {
 // the weight-side sums formed ahead of the call.
 struct Call {
     hipStream_t stream = nullptr;
-    int stages = kAllStages;
+    int stages = kDefaultStages;
     int force_tile = 0;
     BiasEpilogue bias;
     PreparedSums prep;
@@ -611,6 +621,123 @@ static bool fast_shape(int dt, int64_t Mh, int64_t Nh, int64_t Kh) {
     return dt != STHIP_F32 && Mh > 0 && Nh > 0 && Kh > 0 && Mh % 128 == 0 && Nh % 128 == 0 && Kh % kBK2 == 0;
 }
 
+__global__ void clear_flags5_kernel(unsigned* flags) {
+    if (threadIdx.x < kFlagWords) flags[threadIdx.x] = 0;
+}
+
+// One Strassen level as ONE launch (sthip_kernel5.hpp).  Same workspace layout, same arithmetic and
+// same bits as the three-launch form: five sums per operand, seven 16-bit products, fp32 recombination.
+// Run order of the products: M3 M5 M2 M4 M1 M7 M6, so that C12 and C21 are complete after the second
+// and the fourth product and recombine while the later products run; C11 and C22 follow at the end.
+static int one_level_fused(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh, int dt,
+                           bool a_kc, bool b_kc, char* ws, Call& cx) {
+    const LaunchTable5* t5 = table5_for(dt);
+    if (!t5) return 1;
+    const int64_t a_ld = a_kc ? A.rs : A.cs, b_ld = b_kc ? B.cs : B.rs;
+    const size_t sa_b = align256(Mh * Kh * 2), sb_b = align256(Kh * Nh * 2), pm_b = align256(Mh * Nh * 2);
+    char* SA = ws;
+    char* SB = ws + 5 * sa_b;
+    char* PM = ws + 5 * (sa_b + sb_b);
+    unsigned* flags = reinterpret_cast<unsigned*>(ws + prepass_body_bytes(1, Mh, Nh, Kh));
+    const int64_t sa_ld = a_kc ? Kh : Mh, sb_ld = b_kc ? Kh : Nh;
+    const char* Aq[4]; const char* Bq[4];
+    for (int q = 0; q < 4; ++q) {
+        Aq[q] = A.p + ((int64_t)(q >> 1) * Mh * A.rs + (int64_t)(q & 1) * Kh * A.cs) * 2;
+        Bq[q] = B.p + ((int64_t)(q >> 1) * Kh * B.rs + (int64_t)(q & 1) * Nh * B.cs) * 2;
+    }
+    Fused5Params P;
+    memset(&P, 0, sizeof(P));
+    auto SAo = [&](int o) { return (const void*)(SA + (size_t)o * sa_b); };
+    auto SBo = [&](int o) { return (const void*)(SB + (size_t)o * sb_b); };
+    // products in run order; A sums S2 S3 S5 S7 S9 = SA 0..4, B sums S1 S4 S6 S8 S10 = SB 0..4
+    P.g.seg[0] = Seg2{Aq[0], SBo(0), a_ld, sb_ld, 0, 0};     // M3 = A11 S1
+    P.g.seg[1] = Seg2{SAo(0), Bq[3], sa_ld, b_ld, 0, 0};     // M5 = S2 B22
+    P.g.seg[2] = Seg2{SAo(1), Bq[0], sa_ld, b_ld, 0, 0};     // M2 = S3 B11
+    P.g.seg[3] = Seg2{Aq[3], SBo(1), a_ld, sb_ld, 0, 0};     // M4 = A22 S4
+    P.g.seg[4] = Seg2{SAo(2), SBo(2), sa_ld, sb_ld, 0, 0};   // M1 = S5 S6
+    P.g.seg[5] = Seg2{SAo(3), SBo(3), sa_ld, sb_ld, 0, 0};   // M7 = S7 S8
+    P.g.seg[6] = Seg2{SAo(4), SBo(4), sa_ld, sb_ld, 0, 0};   // M6 = S9 S10
+    P.g.C = PM; P.g.c_rs = Nh; P.g.c_ps = (int64_t)(pm_b / 2); P.g.c_bs = 0;
+    P.g.Mh = (int)Mh; P.g.Nh = (int)Nh; P.g.Kh = (int)Kh;
+    P.g.tiles_m = (int)(Mh / kBM4); P.g.tiles_n = (int)(Nh / kBN4);
+    P.g.group_m = 4; P.g.nprod = 7; P.g.c_wide = 1;
+    const int streaming = streaming_hint(prepass_bytes(1, Mh, Nh, Kh));
+    P.g.c_stream = 0; P.streaming = streaming;   // the tiles are read again by the recombination items of this launch
+    P.tiles = P.g.tiles_m * P.g.tiles_n;
+    P.flags = flags;
+    P.c_rs = c_rs; P.rec_rows = (int)Mh; P.rec_chunks = (int)(Nh / 8);
+
+    // element-wise work is cut into units of about 2.5 MB (half the time of a tile at the ~50 GB/s one
+    // CU streams); what must be complete before anything else can start runs on every CU at once
+    auto units_for = [](double bytes) { return (int)std::max<int64_t>(8, round_up((int64_t)(bytes / 2.5e6), 8)); };
+    const int everywhere = 256;
+    auto fill_job = [&](SumJob5& J, bool a_side, const int* outs, int nout, int units) {
+        const int64_t r_ext = a_side ? (a_kc ? Mh : Kh) : (b_kc ? Nh : Kh);
+        const int64_t c_ext = a_side ? (a_kc ? Kh : Mh) : (b_kc ? Kh : Nh);
+        J.ld_in = a_side ? a_ld : b_ld; J.ld_out = a_side ? sa_ld : sb_ld;
+        J.rows = (int)r_ext; J.chunks_per_row = (int)(c_ext / 8); J.nout = nout;
+        J.units = (int)std::min<int64_t>(units, r_ext);
+        bool used[4] = {false, false, false, false};
+        for (int o = 0; o < nout; ++o) {
+            J.out[o] = a_side ? SA + (size_t)outs[o] * sa_b : SB + (size_t)outs[o] * sb_b;
+            for (int q = 0; q < 4; ++q) {
+                J.coef[o][q] = a_side ? kStrA[outs[o]][q] : kStrB[outs[o]][q];
+                if (J.coef[o][q]) used[q] = true;
+            }
+        }
+        for (int q = 0; q < 4; ++q) J.q[q] = used[q] ? (a_side ? Aq[q] : Bq[q]) : nullptr;
+    };
+    const double a_blk = (double)Mh * Kh * 2, b_blk = (double)Kh * Nh * 2, c_blk = (double)Mh * Nh * 2;
+    static const int kS1[1] = {0}, kAall[5] = {0, 1, 2, 3, 4}, kBrest[4] = {1, 2, 3, 4};
+    fill_job(P.job[0], false, kS1, 1, everywhere);
+    fill_job(P.job[1], true, kAall, 5, units_for(9 * a_blk));
+    fill_job(P.job[2], false, kBrest, 4, units_for(8 * b_blk));
+    P.njobs = 3;
+    auto prod_ptr = [&](int p) { return (const void*)(PM + (size_t)p * pm_b); };
+    auto fill_rec = [&](RecJob5& R, int quad, std::initializer_list<int> prods, std::initializer_list<int> signs, int units) {
+        int t = 0;
+        for (int p : prods) R.m[t++] = prod_ptr(p);
+        t = 0;
+        for (int sg : signs) R.sign[t++] = (signed char)sg;
+        R.nterms = (int)prods.size();
+        R.c = C + ((int64_t)(quad >> 1) * Mh * c_rs + (int64_t)(quad & 1) * Nh) * 2;
+        R.units = (int)std::min<int64_t>(units, Mh);
+    };
+    fill_rec(P.rec[0], 1, {0, 1}, {1, 1}, units_for(3 * c_blk));                 // C12 = M3 + M5
+    fill_rec(P.rec[1], 2, {2, 3}, {1, 1}, units_for(3 * c_blk));                 // C21 = M2 + M4
+    fill_rec(P.rec[2], 0, {4, 3, 1, 5}, {1, 1, -1, 1}, everywhere);              // C11 = M1 + M4 - M5 + M7
+    fill_rec(P.rec[3], 3, {4, 2, 0, 6}, {1, -1, 1, 1}, everywhere);              // C22 = M1 - M2 + M3 + M6
+
+    int n = 0, next = 0;
+    auto add = [&](int kind, int arg, int count, unsigned need_jobs, unsigned need_prods) {
+        P.item[n] = Item5{next, kind, arg, need_jobs, need_prods};
+        next += (int)round_up(count, 8);   // the XCD of a workgroup is its index modulo eight: keep items aligned
+        ++n;
+    };
+    add(kItemSums, 0, P.job[0].units, 0, 0);
+    add(kItemSums, 1, P.job[1].units, 0, 0);
+    add(kItemTiles, 0, P.tiles, 1u << 0, 0);
+    add(kItemSums, 2, P.job[2].units, 0, 0);
+    add(kItemTiles, 1, P.tiles, 1u << 1, 0);
+    add(kItemTiles, 2, P.tiles, 1u << 1, 0);
+    add(kItemRecombine, 0, P.rec[0].units, 0, (1u << 0) | (1u << 1));
+    add(kItemTiles, 3, P.tiles, 1u << 2, 0);
+    add(kItemTiles, 4, P.tiles, (1u << 1) | (1u << 2), 0);
+    add(kItemRecombine, 1, P.rec[1].units, 0, (1u << 2) | (1u << 3));
+    add(kItemTiles, 5, P.tiles, (1u << 1) | (1u << 2), 0);
+    add(kItemTiles, 6, P.tiles, (1u << 1) | (1u << 2), 0);
+    add(kItemRecombine, 2, P.rec[2].units, 0, (1u << 4) | (1u << 3) | (1u << 1) | (1u << 5));
+    add(kItemRecombine, 3, P.rec[3].units, 0, (1u << 4) | (1u << 2) | (1u << 0) | (1u << 6));
+    P.nitems = n;
+
+    hipLaunchKernelGGL(clear_flags5_kernel, dim3(1), dim3(64), 0, cx.stream, flags);
+    int rc = check_launch("clear_flags");
+    if (rc) return rc;
+    hipError_t e = t5->fn[b_kc ? 1 : 0](P, next, cx.stream);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return STHIP_OK;
+}
+
 // The pipelined path: optional quadrant-sum pre-pass into `ws`, then one grouped-GEMM launch.
 // Returns 1 if the problem does not qualify (the caller then takes the fused kernel).
 static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch, int64_t a_bs, int64_t b_bs,
@@ -631,6 +758,48 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         Aq[q] = A.p + ((int64_t)(q >> 1) * Mh * A.rs + (int64_t)(q & 1) * Kh * A.cs) * 2;
         Bq[q] = B.p + ((int64_t)(q >> 1) * Kh * B.rs + (int64_t)(q & 1) * Nh * B.cs) * 2;
     }
+    // Fixed tile table.  Bytes moved L2 -> LDS per flop go with 1/BM + 1/BN, so the largest tile
+    // that still gives every CU work wins.  256 x 256 holds one accumulator per wave and nothing
+    // else: a classical product runs on it directly, a Strassen / Winograd level runs its seven
+    // products on it as one grouped launch into 16-bit product matrices (the reference's own
+    // cast schedule) followed by the recombination pass.  256 x 128 (two accumulators in
+    // registers, one parked) and 128 x 128 (three in registers) recombine in registers and serve
+    // fp32 results and the sizes that are too small for the large tile.  The large tiles need A
+    // contiguous along k; the recombination pass needs 16-byte aligned rows of C.
+    const LaunchTable3* t3 = table3_for(dt, algo);
+    const LaunchTable3* t4 = table4_for(dt);
+    const int force = cx.force_tile;
+    const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
+    // products as matrices + recombination pass: 16-bit products for a result in the operand type,
+    // fp32 products (twice the room) for an fp32 result
+    const bool f32_prod = split && out_f32 && c_rs % 4 == 0 && c_bs % 4 == 0 && aligned_to(C, 16) &&
+                          ws_bytes >= prepass_bytes(batch, Mh, Nh, Kh, 4);
+    const bool grouped_ok = !split || (out_f32 ? f32_prod : c_vec);
+    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && grouped_ok;
+    const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
+    const bool can5 = split && !out_f32 && grouped_ok;
+    const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch * (split ? 7 : 1);
+    const int64_t tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
+    const int64_t tiles2 = (Mh / 128) * (Nh / 128) * batch;
+    // Measured on MI355X (bf16): the 256 x 256 grouped path wins from 4096^3 up when k is long
+    // enough to pay for writing the sums and the products (its extra passes cost bytes
+    // ~ MK + KN + MN, the products flops ~ MNK); when the 128 x 128 tiles of ONE product cannot
+    // fill the 256 CUs (small matrices, weight gradients with short M and N) the seven products
+    // side by side can, and that launch is 2 - 4 x faster; otherwise recombining in registers
+    // (no product round trip) is as fast or faster.
+    int pick = 2;
+    if (can4 && tiles4 >= (split ? 400 : 224) && (!split || Kh >= 1024)) pick = 4;
+    else if (can5 && tiles2 < 256) pick = 5;
+    else if (can3 && tiles3 >= 256) pick = 3;
+    if (force == 4 && can4) pick = 4;
+    else if (force == 3 && can3) pick = 3;
+    else if (force == 5 && can5) pick = 5;
+    else if (force == 2) pick = 2;
+    // one level on the large tile, plain result in the operand type: everything as work items of one launch
+    if (pick == 4 && split && algo == STHIP_STRASSEN && !out_f32 && !accumulate && batch == 1 && (cx.stages & 16) &&
+        (cx.stages & 7) == 7 && !(cx.bias.bias && cx.bias.target == C) && !cx.prep.sums && table5_for(dt))
+        return one_level_fused(A, B, C, c_rs, Mh, Nh, Kh, dt, a_kc, b_kc, ws, cx);
+    hipError_t e = hipSuccess;
     if (!split) {
         p.seg[0] = {A.p, B.p, a_ld, b_ld, a_bs, b_bs};
     } else {
@@ -699,44 +868,6 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
             set(6, Aq[3], a_ld, a_bs, SBo(3), sb_ld, sb_bs);      // -P4 = A22 (-T4)
         }
     }
-    // Fixed tile table.  Bytes moved L2 -> LDS per flop go with 1/BM + 1/BN, so the largest tile
-    // that still gives every CU work wins.  256 x 256 holds one accumulator per wave and nothing
-    // else: a classical product runs on it directly, a Strassen / Winograd level runs its seven
-    // products on it as one grouped launch into 16-bit product matrices (the reference's own
-    // cast schedule) followed by the recombination pass.  256 x 128 (two accumulators in
-    // registers, one parked) and 128 x 128 (three in registers) recombine in registers and serve
-    // fp32 results and the sizes that are too small for the large tile.  The large tiles need A
-    // contiguous along k; the recombination pass needs 16-byte aligned rows of C.
-    hipError_t e = hipSuccess;
-    const LaunchTable3* t3 = table3_for(dt, algo);
-    const LaunchTable3* t4 = table4_for(dt);
-    const int force = cx.force_tile;
-    const bool c_vec = c_rs % 8 == 0 && c_bs % 8 == 0 && aligned_to(C, 16);
-    // products as matrices + recombination pass: 16-bit products for a result in the operand type,
-    // fp32 products (twice the room) for an fp32 result
-    const bool f32_prod = split && out_f32 && c_rs % 4 == 0 && c_bs % 4 == 0 && aligned_to(C, 16) &&
-                          ws_bytes >= prepass_bytes(batch, Mh, Nh, Kh, 4);
-    const bool grouped_ok = !split || (out_f32 ? f32_prod : c_vec);
-    const bool can4 = a_kc && Mh % kBM4 == 0 && Nh % kBN4 == 0 && t4 && grouped_ok;
-    const bool can3 = a_kc && Mh % kBM3 == 0 && t3;
-    const bool can5 = split && !out_f32 && grouped_ok;
-    const int64_t tiles4 = (Mh / kBM4) * (Nh / kBN4) * batch * (split ? 7 : 1);
-    const int64_t tiles3 = (Mh / kBM3) * (Nh / kBN3) * batch;
-    const int64_t tiles2 = (Mh / 128) * (Nh / 128) * batch;
-    // Measured on MI355X (bf16): the 256 x 256 grouped path wins from 4096^3 up when k is long
-    // enough to pay for writing the sums and the products (its extra passes cost bytes
-    // ~ MK + KN + MN, the products flops ~ MNK); when the 128 x 128 tiles of ONE product cannot
-    // fill the 256 CUs (small matrices, weight gradients with short M and N) the seven products
-    // side by side can, and that launch is 2 - 4 x faster; otherwise recombining in registers
-    // (no product round trip) is as fast or faster.
-    int pick = 2;
-    if (can4 && tiles4 >= (split ? 400 : 224) && (!split || Kh >= 1024)) pick = 4;
-    else if (can5 && tiles2 < 256) pick = 5;
-    else if (can3 && tiles3 >= 256) pick = 3;
-    if (force == 4 && can4) pick = 4;
-    else if (force == 3 && can3) pick = 3;
-    else if (force == 5 && can5) pick = 5;
-    else if (force == 2) pick = 2;
     if ((pick == 4 || pick == 5) && split) {
         Recombine16Params rp;
         rp.prod = p.park; rp.C = C; rp.c_rs = c_rs; rp.c_bs = c_bs;

@@ -6,6 +6,7 @@
 #include "sthip_kernel2.hpp"
 #include "sthip_kernel3.hpp"
 #include "sthip_kernel4.hpp"
+#include "sthip_kernel5.hpp"
 
 namespace sthip {
 
@@ -102,6 +103,23 @@ hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
     const int nprod = p.nprod > 0 ? p.nprod : 1;
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
     hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, p);
+    return hipGetLastError();
+}
+
+// One-launch Strassen level (16-bit operands, A contiguous along k): tables indexed [b_kc]; `blocks`
+// is the length of the work-item list.
+typedef hipError_t (*LaunchFn5)(const Fused5Params&, int blocks, hipStream_t);
+struct LaunchTable5 { LaunchFn5 fn[2]; };
+extern const LaunchTable5 kLaunch5_1;
+extern const LaunchTable5 kLaunch5_2;
+
+template <class T, bool B_KC>
+hipError_t launch_fused5(const Fused5Params& p, int blocks, hipStream_t stream) {
+    auto kern = fused5_kernel<T, B_KC>;
+    static OptIn opted;
+    hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes4);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads4), kSmemBytes4, stream, p);
     return hipGetLastError();
 }
 

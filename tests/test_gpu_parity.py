@@ -461,3 +461,33 @@ def test_fp32_two_levels_flat_against_host_recursion(hip, tb):
     want = A.double() @ B.double()
     err = float(torch.linalg.norm(fused.cpu().double() - want) / torch.linalg.norm(want))
     assert err <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,tb", [((4096, 4096, 4096), False), ((4096, 4096, 4096), True), ((4096, 8192, 2048), True),
+                                      ((4096, 6144, 4096), False)])
+def test_one_level_as_one_launch_same_bits(hip, dtype, shape, tb):
+    """Bit 4 of the debug stage mask runs a large one-level call as ONE launch whose workgroups are
+    the sums, the product tiles and the recombination, ordered by counters in the workspace.  Same
+    arithmetic in the same order as the three launches, so the same bits -- also when the workspace
+    is reused with other inputs (a stale sum or product from the previous call would show), and no
+    workgroup may have given up waiting."""
+    from strassen_hip import _capi
+    lib = _capi.load()
+    M, N, K = shape
+    A = _gauss((M, K), 201, K ** -0.5, dtype).cuda()
+    B = _layout(_gauss((K, N), 202, 1.0, dtype), tb)
+    ws = torch.empty(hip.workspace_bytes(A, B, levels=1), dtype=torch.uint8, device="cuda")
+    for rep in range(3):
+        want = hip.gemm(A, B, levels=1, workspace=ws).clone()
+        prev = lib.sthip_debug_set_stages(31)
+        try:
+            got = hip.gemm(A, B, levels=1, workspace=ws)
+            torch.cuda.synchronize()
+        finally:
+            lib.sthip_debug_set_stages(prev)
+        counters = ws[-256:].view(torch.int32)[:16].tolist()
+        assert counters[15] == 0, counters                       # nobody gave up
+        assert counters[8:15] == [(M // 512) * (N // 512)] * 7   # the one-launch form did run: every tile counted
+        assert torch.equal(got, want), rep
+        A = (A * -0.5 + 0.125).to(dtype)

@@ -70,11 +70,11 @@ def test_argument_errors_need_no_gpu():
     assert b"no unit stride" in lib.sthip_last_error()
     # workspace.  One level: room for the ten quadrant sums (5 per operand) and the parked accumulator when the shape is
     # tile aligned, per batch entry; nothing for fp32, odd or unaligned shapes, or classic.
-    sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles)
+    sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 2 + 256   # ten 16-bit sums + seven 16-bit products (or parked fp32 tiles) + counters
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 1) == sums(512)
     assert lib.sthip_workspace_bytes(3, 1024, 1024, 1024, 1, 1, 2, 1) == 3 * sums(512)
     # 16-bit operands with an fp32 result: the seven products stay fp32
-    assert lib.sthip_workspace_bytes(2, 1024, 1024, 1024, 2, 0, 1, 1) == 2 * (2 * 5 * 512 * 512 * 2 + 7 * 512 * 512 * 4)
+    assert lib.sthip_workspace_bytes(2, 1024, 1024, 1024, 2, 0, 1, 1) == 2 * (2 * 5 * 512 * 512 * 2 + 7 * 512 * 512 * 4) + 256
     # fp32, tile aligned: seven dense A operands, seven B operands, seven fp32 products
     f32 = lambda h: 7 * 3 * h * h * 4
     assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 1) == f32(512)
@@ -88,7 +88,7 @@ def test_argument_errors_need_no_gpu():
     # launch -- ten half-size sums, 70 quarter-size sums and 49 quarter-size products; the query covers
     # whichever is larger.
     upper = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
-    inner_sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4
+    inner_sums = lambda h: 2 * 5 * h * h * 2 + 7 * h * h * 4 + 256
     flat = lambda h: 10 * h * h * 2 + (70 + 49) * (h // 2) ** 2 * 2
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
     assert two == max(upper(512) + inner_sums(256), flat(512))
