@@ -182,7 +182,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="strassen1_8192_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--force-tile", default=None, choices=["128x128", "128x128g", "256x128", "256x256"],
+    ap.add_argument("--force-tile", default=None, choices=["128x128", "128x128g", "256x128", "256x256", "64x64"],
                     help="override the library's tile table (STHIP_FORCE_TILE): 256x128 and 128x128 are the "
                          "kernels that recombine in registers, 128x128g / 256x256 the grouped paths")
     args = ap.parse_args()

@@ -26,7 +26,8 @@ int sthip_debug_transpose_read(void* out, void* stream);
 int sthip_debug_set_stages(int mask);
 
 /* Overrides the tile table for later calls where the shape allows the forced tile: "128x128",
- * "256x128" (kernels that recombine in registers), "128x128g", "256x256" (grouped products);
+ * "256x128" (kernels that recombine in registers), "128x128g", "256x256" (grouped products),
+ * "64x64" (fp32: seven products side by side on small tiles, sums formed in the operand loads);
  * NULL or anything else = automatic.  Returns the previous setting as a code (0 = automatic).
  * The environment variable STHIP_FORCE_TILE gives the initial setting; it is read once, by the
  * first call into the library. */

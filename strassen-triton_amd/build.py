@@ -45,6 +45,7 @@ def _units():
         units.append((f"sthip_inst4_{t}.o", "sthip_inst4.hip", [f"-DSTHIP_INST_TYPE={t}"]))
         units.append((f"sthip_inst5_{t}.o", "sthip_inst5.hip", [f"-DSTHIP_INST_TYPE={t}"]))
     units.append(("sthip_inst4_0.o", "sthip_inst4.hip", ["-DSTHIP_INST_TYPE=0"]))
+    units.append(("sthip_inst6.o", "sthip_inst6.hip", []))
     return units
 
 

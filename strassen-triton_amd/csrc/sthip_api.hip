@@ -87,7 +87,7 @@ static const LaunchTable3* table4_for(int dt) {
     return dt == STHIP_F32 ? &kLaunch4_0 : dt == STHIP_F16 ? &kLaunch4_1 : dt == STHIP_BF16 ? &kLaunch4_2 : nullptr;
 }
 
-// STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 in the environment of the process overrides the
+// STHIP_FORCE_TILE=128x128 | 128x128g | 256x128 | 256x256 | 64x64 in the environment of the process overrides the
 // tile table where the shape allows the forced tile (tuning aid); it is read once, by the first call.
 // sthip_debug_force_tile changes the setting later.
 static int tile_code(const char* e) {
@@ -96,6 +96,7 @@ static int tile_code(const char* e) {
     if (!strcmp(e, "256x128")) return 3;
     if (!strcmp(e, "256x256")) return 4;
     if (!strcmp(e, "128x128g")) return 5;   // 128 x 128 tiles, seven products as separate outputs
+    if (!strcmp(e, "64x64")) return 6;      // fp32: 64 x 64 tiles, seven products side by side, sums formed in the loads
     return 0;
 }
 static int forced_tile_setting() {
@@ -935,6 +936,9 @@ static int one_level_f32_batched(View A, View B, char* C, int64_t c_rs, int64_t 
                                  bool accumulate, char* ws, Call& cx);
 static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
                                  int algo, bool accumulate, char* ws, Call& cx);
+static bool f32_small_shape(View A, View B, int64_t Mh, int64_t Nh, int64_t Kh);
+static int one_level_f32_small(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
+                               bool accumulate, char* ws, Call& cx);
 
 static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                         int64_t batch, int64_t a_bs, int64_t b_bs, int64_t c_bs,
@@ -1012,12 +1016,31 @@ static int launch_fused(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
             ws_bytes >= f32_batched_bytes(Mh, Nh, Kh))
             return one_level_f32_grouped(A, B, C, c_rs, Mh, Nh, Kh, algo, accumulate, ws, cx);
     }
+    // fp32 classical product too small for the 256 x 256 kernel: 64 x 64 tiles (sthip_kernel6.hpp, one
+    // product, no sums).  Measured against the 128 x 128 fused kernel: 1024^3 0.098 -> 0.03 ms.
+    if (fast && dt == STHIP_F32 && !split && batch == 1 && cx.force_tile != 2 && f32_small_shape(A, B, Mh, Nh, Kh)) {
+        Gemm6Params g;
+        memset(&g, 0, sizeof(g));
+        g.a[0] = Op6{reinterpret_cast<const float*>(A.p), nullptr, A.rs, 0, 0};
+        g.b[0] = Op6{reinterpret_cast<const float*>(B.p), nullptr, b_kc ? B.cs : B.rs, 0, 0};
+        g.C = reinterpret_cast<float*>(C); g.c_rs = c_rs; g.c_ps = 0;
+        g.Kh = (int)Kh; g.tiles_m = (int)(Mh / kBM6); g.tiles_n = (int)(Nh / kBN6); g.nprod = 1;
+        g.accumulate = accumulate ? 1 : 0;
+        hipError_t e = launch_gemm6(g, b_kc, cx.stream);
+        if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+        return STHIP_OK;
+    }
     // fp32, one Strassen level: run the seven products side by side as a batch (see
     // one_level_f32_batched).  Measured against the fused kernel: 5 x faster at 1024^3 (one product
     // has 16 tiles for 256 CUs), 3 x at 2048^3, equal at 4096^3, 10 % faster at 8192^3.
     if (fast && dt == STHIP_F32 && algo == STHIP_STRASSEN && batch == 1 && ws && aligned_to(ws, 256) &&
-        ws_bytes >= f32_batched_bytes(Mh, Nh, Kh) && cx.force_tile != 2)
+        ws_bytes >= f32_batched_bytes(Mh, Nh, Kh) && cx.force_tile != 2) {
+        // small products: 64 x 64 tiles with the sums formed in the operand loads (two launches);
+        // measured against the batched form below: see one_level_f32_small
+        if (f32_small_shape(A, B, Mh, Nh, Kh) && (cx.force_tile == 6 || (cx.force_tile == 0 && Mh * Nh <= (int64_t)1024 * 1024)))
+            return one_level_f32_small(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, cx);
         return one_level_f32_batched(A, B, C, c_rs, Mh, Nh, Kh, accumulate, ws, cx);
+    }
     const LaunchTable* t = table_for(dt, algo);
     if (!t) return fail(STHIP_ERR_ARG, "bad dtype/algo (%d, %d)", dt, algo);
     hipError_t e = t->fn[a_kc ? 1 : 0][b_kc ? 1 : 0][fast ? 0 : 1](p, (int)batch, cx.stream);
@@ -1498,6 +1521,39 @@ struct Term { int a, b, sign; };
 static const Term kATerms[7] = {{0, 3, +1}, {2, 3, +1}, {0, 0, 0}, {3, 0, 0}, {0, 1, +1}, {2, 0, -1}, {1, 3, -1}};
 static const Term kBTerms[7] = {{0, 3, +1}, {0, 0, 0}, {1, 3, -1}, {2, 0, -1}, {3, 0, 0}, {0, 1, +1}, {2, 3, +1}};
 
+// fp32, one Strassen level on small matrices: the seven products side by side on 64 x 64 tiles, every
+// operand a quadrant read in place or the sum / difference of two formed in registers on the way
+// to LDS (sthip_kernel6.hpp), then the recombination pass.  Two launches instead of three and 7 x
+// (Mh / 64) x (Nh / 64) workgroups instead of 7 x (Mh / 128) x (Nh / 128).
+static bool f32_small_shape(View A, View B, int64_t Mh, int64_t Nh, int64_t Kh) {
+    if (A.cs != 1 || (B.rs != 1 && B.cs != 1)) return false;
+    if (Mh % kBM6 || Nh % kBN6 || Kh % (2 * kBK6)) return false;
+    const int64_t b_ld = B.rs == 1 ? B.cs : B.rs;
+    return aligned_to(A.p, 16) && aligned_to(B.p, 16) && A.rs % 4 == 0 && b_ld % 4 == 0;
+}
+static int one_level_f32_small(View A, View B, char* C, int64_t c_rs, int64_t Mh, int64_t Nh, int64_t Kh,
+                               bool accumulate, char* ws, Call& cx) {
+    const size_t sm = align256(Mh * Nh * 4);
+    const bool b_kc = B.rs == 1;
+    Gemm6Params g;
+    memset(&g, 0, sizeof(g));
+    const float* Aq[4]; const float* Bq[4];
+    for (int q = 0; q < 4; ++q) {
+        Aq[q] = reinterpret_cast<const float*>(A.p) + (int64_t)(q >> 1) * Mh * A.rs + (int64_t)(q & 1) * Kh * A.cs;
+        Bq[q] = reinterpret_cast<const float*>(B.p) + (int64_t)(q >> 1) * Kh * B.rs + (int64_t)(q & 1) * Nh * B.cs;
+    }
+    for (int q = 0; q < 7; ++q) {
+        g.a[q] = Op6{Aq[kATerms[q].a], Aq[kATerms[q].b], A.rs, kATerms[q].sign, 0};
+        g.b[q] = Op6{Bq[kBTerms[q].a], Bq[kBTerms[q].b], b_kc ? B.cs : B.rs, kBTerms[q].sign, 0};
+    }
+    g.C = reinterpret_cast<float*>(ws); g.c_rs = Nh; g.c_ps = (int64_t)(sm / 4);
+    g.Kh = (int)Kh; g.tiles_m = (int)(Mh / kBM6); g.tiles_n = (int)(Nh / kBN6); g.nprod = 7;
+    hipError_t e = launch_gemm6(g, b_kc, cx.stream);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+    return recombine(STHIP_F32, C, c_rs, 1, reinterpret_cast<const float*>(ws), (int64_t)(sm / 4), Mh, Nh, 2 * Mh, 2 * Nh,
+                     accumulate, cx.stream);
+}
+
 // sums by product M1..M7 as indices into the outputs of kStrA / kStrB (-1 = a raw block)
 static const int kSumA[7] = {2, 1, -1, -1, 0, 4, 3};
 static const int kSumB[7] = {2, -1, 0, 1, -1, 4, 3};
@@ -1766,7 +1822,6 @@ static int auto_levels(int64_t M, int64_t N, int64_t K, int dt, int max_levels) 
     if (max_levels <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
     const int64_t smallest = std::min(M, std::min(N, K));
     const double flops = 2.0 * (double)M * (double)N * (double)K;
-    const int64_t tiles256 = ceil_div(M, 256) * ceil_div(N, 256);
     int levels = 0;
     if (dt == STHIP_F32) {
         // the fp32 matrix cores are 16 x slower than the 16-bit ones while the passes only double:
@@ -1775,10 +1830,9 @@ static int auto_levels(int64_t M, int64_t N, int64_t K, int dt, int max_levels) 
         if (std::min(M, N) >= 4096 && K >= 4096 && flops >= 5e11) levels = 1;
         if (smallest >= 4096 && flops >= 1e12) levels = 2;
         if (smallest >= 32768) levels = 3;
-        // fewer than 224 tiles of 256 x 256: the classical product runs on the 128 x 128 kernel, the
-        // seven half-size products of a level fill the large-tile kernel or run as one batch (1.3 - 1.8 x)
-        if (levels == 0 && tiles256 < 224 && M >= 1024 && N >= 1024 && K >= 1024 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0)
-            levels = 1;
+        // fewer than 224 tiles of 256 x 256: the classical product runs on 64 x 64 tiles at 0.8 - 0.9 x
+        // hipBLASLt, and a level on top of it is 0.75 - 1.0 x of that up to k = 4096 (1.01 - 1.05 x beyond):
+        // classical
     } else {
         // 16-bit: the passes of a level cost about 14 n^2 bytes against n^3 / 4 flop saved: break-even
         // near 16384^3 (1.02 - 1.05 x there, 0.92 x at 8192^3); a second level from 32768^3, a third from 65536^3

@@ -7,6 +7,7 @@
 #include "sthip_kernel3.hpp"
 #include "sthip_kernel4.hpp"
 #include "sthip_kernel5.hpp"
+#include "sthip_kernel6.hpp"
 
 namespace sthip {
 
@@ -122,5 +123,8 @@ hipError_t launch_fused5(const Fused5Params& p, int blocks, hipStream_t stream) 
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads4), kSmemBytes4, stream, p);
     return hipGetLastError();
 }
+
+// 64 x 64 fp32 kernel with the pre-additions fused into the loads (defined in sthip_inst6.hip).
+hipError_t launch_gemm6(const Gemm6Params& p, bool b_kc, hipStream_t stream);
 
 }  // namespace sthip

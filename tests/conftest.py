@@ -42,7 +42,7 @@ def force_tile():
     test ends; the previous setting comes back afterwards."""
     from strassen_hip import _capi
     lib = _capi.load()
-    names = {0: None, 2: b"128x128", 3: b"256x128", 4: b"256x256", 5: b"128x128g"}
+    names = {0: None, 2: b"128x128", 3: b"256x128", 4: b"256x256", 5: b"128x128g", 6: b"64x64"}
     first = []
 
     def force(tile):

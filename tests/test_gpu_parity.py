@@ -304,6 +304,32 @@ def test_fp32_batched_products(hip, force_tile, ta, tb, shape):
     assert rel(acc, ref + C0.double()) <= 1e-5
 
 
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 128), (512, 256, 640), (1024, 1024, 1024), (2048, 1024, 512)])
+def test_fp32_small_tiles(hip, force_tile, tb, shape):
+    """fp32 on 64 x 64 tiles: one Strassen level with the quadrant sums formed in the operand loads
+    (seven products side by side, then the recombination pass), and the plain classical product.
+    Exact on integers, also when accumulating; on Gaussian inputs within 1e-5 of fp64 (the
+    configuration's bound for fp32) and of the batched three-launch form."""
+    M, N, K = shape
+    A, B, C0 = _ints((M, K), 71), _ints((K, N), 72), _ints((M, N), 73)
+    Ag, Bg = A.cuda(), _layout(B, tb)
+    want = A.double() @ B.double()
+    force_tile("64x64")
+    assert torch.equal(hip.gemm(Ag, Bg, algo="strassen", levels=1).cpu().double(), want)
+    assert torch.equal(hip.gemm(Ag, Bg, out=C0.cuda(), algo="strassen", levels=1, accumulate=True).cpu().double(), want + C0.double())
+    assert torch.equal(hip.gemm(Ag, Bg, algo="classic", levels=0).cpu().double(), want)
+    assert torch.equal(hip.gemm(Ag, Bg, out=C0.cuda(), algo="classic", levels=0, accumulate=True).cpu().double(), want + C0.double())
+    A, B = _gauss((M, K), 74, 1.0, torch.float32), _gauss((K, N), 75, 1.0, torch.float32)
+    Ag, Bg = A.cuda(), _layout(B, tb)
+    small, classic = hip.gemm(Ag, Bg, algo="strassen", levels=1), hip.gemm(Ag, Bg, algo="classic", levels=0)
+    force_tile("128x128g")
+    batched = hip.gemm(Ag, Bg, algo="strassen", levels=1)
+    ref = A.double() @ B.double()
+    rel = lambda X, R: float(torch.linalg.norm(X.cpu().double() - R) / torch.linalg.norm(R))
+    assert rel(small, ref) <= 1e-5 and rel(classic, ref) <= 1e-5 and rel(small, batched.cpu().double()) <= 1e-5
+
+
 def _sweep_cases():
     import itertools
     import random
