@@ -115,6 +115,19 @@ static int wide_rows(const void* C, int64_t rs, int64_t ps, int64_t bs) {
     return aligned_to(C, 16) && rs % 8 == 0 && ps % 8 == 0 && bs % 8 == 0 ? 1 : 0;
 }
 
+// Quadrant sums as coefficients over (X11, X12, X21, X22).  Strassen (fixed_strassen.py:88-97): A side
+// S2 S3 S5 S7 S9, B side S1 S4 S6 S8 S10.  Winograd: A side S1 S2 S3 S4; B side T1 T2 T3 -T4.
+constexpr int str_coef(int side, int o, int q) {
+    constexpr signed char a[5][4] = {{1, 1, 0, 0}, {0, 0, 1, 1}, {1, 0, 0, 1}, {0, 1, 0, -1}, {-1, 0, 1, 0}};
+    constexpr signed char b[5][4] = {{0, 1, 0, -1}, {-1, 0, 1, 0}, {1, 0, 0, 1}, {0, 0, 1, 1}, {1, 1, 0, 0}};
+    return side == 0 ? a[o][q] : b[o][q];
+}
+constexpr int win_coef(int side, int o, int q) {
+    constexpr signed char a[4][4] = {{0, 0, 1, 1}, {-1, 0, 1, 1}, {1, 0, -1, 0}, {1, 1, -1, -1}};
+    constexpr signed char b[4][4] = {{-1, 1, 0, 0}, {1, -1, 0, 1}, {0, -1, 0, 1}, {-1, 1, 1, -1}};
+    return side == 0 ? a[o][q] : b[o][q];
+}
+
 // ------------------------------------------------------------------ quadrant-sum pre-pass
 // out[o] = sum_q coef[o][q] * quadrant q, for up to five outputs at once, on matrices seen
 // in storage order (rows x cols, cols contiguous).  Each thread handles one 16-byte chunk
@@ -126,10 +139,15 @@ struct ComboParams {
     int64_t ld_in, bs_in, ld_out, bs_out;   // elements
     int nout, rows, chunks_per_row;
     int streaming;   // loads and stores carry the streaming hint (working set larger than the caches)
+    int table;       // 16-bit kernels: 0 / 1 = the five Strassen sums of an A / B operand, 2 / 3 = the four Winograd sums
+                     // (coefficients compiled in); anything else: coef below
     signed char coef[7][4];
 };
 
-template <class T>
+// TABLE 0..3: coefficients known at compile time (every term a constant, zero terms vanish); -1: read
+// from p.coef.  With run-time coefficients the pass issued 680 VALU instructions per thread and kept the
+// vector ALUs busy 72 % of its time; the products only ever need the four fixed tables.
+template <class T, int TABLE>
 __device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
@@ -149,18 +167,7 @@ __device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
             if constexpr (__is_same(T, bf16_t)) { x[q][2 * w] = bf16lo(word); x[q][2 * w + 1] = bf16hi(word); }
             else { const f16x2 h = as_f16x2(word); x[q][2 * w] = (float)h[0]; x[q][2 * w + 1] = (float)h[1]; }
         }
-    for (int o = 0; o < p.nout; ++o) {
-        float s[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float acc = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int cf = p.coef[o][q];
-                if (cf > 0) acc += x[q][e]; else if (cf < 0) acc -= x[q][e];
-            }
-            s[e] = acc;
-        }
+    auto emit = [&](int o, const float* s) {
         u32x4 w;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -168,11 +175,53 @@ __device__ __forceinline__ void quad_combos_body(const ComboParams& p) {
             else w[i] = pack_f16(s[2 * i], s[2 * i + 1]);
         }
         store_hinted(w, reinterpret_cast<u32x4*>(reinterpret_cast<char*>(p.out[o]) + out_off), p.streaming);
+    };
+    if constexpr (TABLE >= 0) {
+        constexpr int NOUT = TABLE < 2 ? 5 : 4;
+#pragma unroll
+        for (int o = 0; o < NOUT; ++o) {
+            float s[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float acc = 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int cf = TABLE < 2 ? str_coef(TABLE, o, q) : win_coef(TABLE - 2, o, q);
+                    if (cf > 0) acc += x[q][e]; else if (cf < 0) acc -= x[q][e];
+                }
+                s[e] = acc;
+            }
+            emit(o, s);
+        }
+    } else {
+        for (int o = 0; o < p.nout; ++o) {
+            float s[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float acc = 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int cf = p.coef[o][q];
+                    if (cf > 0) acc += x[q][e]; else if (cf < 0) acc -= x[q][e];
+                }
+                s[e] = acc;
+            }
+            emit(o, s);
+        }
     }
+}
+template <class T>
+__device__ __forceinline__ void quad_combos_any(const ComboParams& p) {
+    const int table = __builtin_amdgcn_readfirstlane(p.table);
+    if (table == 0) quad_combos_body<T, 0>(p);
+    else if (table == 1) quad_combos_body<T, 1>(p);
+    else if (table == 2) quad_combos_body<T, 2>(p);
+    else if (table == 3) quad_combos_body<T, 3>(p);
+    else quad_combos_body<T, -1>(p);
 }
 
 template <class T>
-__global__ void __launch_bounds__(256) quad_combos_kernel(const ComboParams p) { quad_combos_body<T>(p); }
+__global__ void __launch_bounds__(256) quad_combos_kernel(const ComboParams p) { quad_combos_any<T>(p); }
 
 // fp32 form: four elements per 16-byte chunk, sums stay fp32 (nothing to round).
 __device__ __forceinline__ void quad_combos_f32_body(const ComboParams& p) {
@@ -197,7 +246,7 @@ __device__ __forceinline__ void quad_combos_f32_body(const ComboParams& p) {
 // Both operands of a level in one launch: blockIdx.z picks the side.
 struct ComboPair { ComboParams side[2]; };
 template <class T>
-__global__ void __launch_bounds__(256) quad_combos_pair_kernel(const ComboPair pp) { quad_combos_body<T>(pp.side[blockIdx.z]); }
+__global__ void __launch_bounds__(256) quad_combos_pair_kernel(const ComboPair pp) { quad_combos_any<T>(pp.side[blockIdx.z]); }
 
 __global__ void __launch_bounds__(256) quad_combos_pair_f32_kernel(const ComboPair pp) { quad_combos_f32_body(pp.side[blockIdx.z]); }
 
@@ -265,19 +314,38 @@ struct Combo2Params {
     int64_t ld_in, ld1, ld2;  // elements
     int64_t q1_u, q1_v;       // element offset of quarter (u, v) inside a first-level sum: u * q1_u + v * q1_v
     int rows, chunks_per_row; // of one quarter block, storage order
-    int nout2, keep;          // second-level sums per operand; quarters (bit 2 u + v) of the first-level sums to store
+    int side;                 // 0: the tables of the A operand, 1: of the B operand
+    int algo2;                // algorithm of the second level (the first is always Strassen)
     int streaming;            // loads and stores carry the streaming hint
-    signed char l1[7][4];     // first-level operand p over the quadrants 11 12 21 22 (a unit vector = that quadrant)
-    signed char l1_sum[7];    // index into s1 if p is a sum, -1 if it is a quadrant
-    signed char c2[5][4];     // second-level sums over the four quarters of a first-level operand
 };
 struct Combo2Pair { Combo2Params side[2]; };
 
-template <class T>
-__global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) {
+// Coefficient tables of the two-level pass, evaluated at compile time: the loops over operands,
+// quarters and terms are unrolled, so every coefficient is a constant and zero terms vanish.  (With the
+// tables as kernel arguments the pass issued 3300 VALU instructions per thread and was bound by them,
+// not by memory: 4.1 TB/s.)
+// First-level operands in the order the 49 products use them: A side A11 S9 S2 S7 S5 S3 A22, B side
+// S1 S10 B22 S8 S6 B11 S4.  >= 0: index of the sum among the five; -1 - q: quadrant q as it is.
+constexpr int first_code(int side, int p) {
+    constexpr signed char a[7] = {-1, 4, 0, 3, 2, 1, -4}, b[7] = {0, 4, -4, 3, 2, -1, 1};
+    return side == 0 ? a[p] : b[p];
+}
+constexpr int first_coef(int side, int p, int q) {
+    const int f = first_code(side, p);
+    return f >= 0 ? str_coef(side, f, q) : (q == -1 - f ? 1 : 0);
+}
+constexpr int second_coef(int side, int algo2, int o, int uv) {
+    return algo2 == STHIP_STRASSEN ? str_coef(side, o, uv) : win_coef(side, o, uv);
+}
+// Quarters (bit 2 u + v) of a first-level sum that the second level multiplies as they are: Strassen
+// 11 and 22; Winograd 11, 12 and 22 of an A-side operand, 11, 21 and 22 of a B-side one.
+constexpr int kept_quarters(int side, int algo2) { return algo2 == STHIP_STRASSEN ? 0x9 : (side == 0 ? 0xB : 0xD); }
+
+template <class T, int SIDE, int ALGO2>
+__device__ __forceinline__ void combos2_body(const Combo2Params& p) {
     typedef typename ElemVec<T>::type vec_t;
     constexpr int ES = (int)sizeof(T) == 4 ? 4 : 2;
-    const Combo2Params& p = pp.side[blockIdx.z];
+    constexpr int NOUT2 = ALGO2 == STHIP_STRASSEN ? 5 : 4;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)p.rows * p.chunks_per_row) return;
     const int r = (int)(idx / p.chunks_per_row), c = (int)(idx % p.chunks_per_row);
@@ -287,39 +355,47 @@ __global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) 
 #pragma unroll
     for (int b = 0; b < 16; ++b)
         v[b] = load_hinted(reinterpret_cast<const vec_t*>(reinterpret_cast<const char*>(p.x[b]) + in_off), p.streaming);
+#pragma unroll
     for (int q = 0; q < 7; ++q) {
-        // quarters (u, v) of first-level operand q
+        // quarters (u, v) of first-level operand q, in the operand type and unpacked
         vec_t s[4];
+        float x[4][kEPT2];
+        const int code = first_code(SIDE, q);
 #pragma unroll
         for (int uv = 0; uv < 4; ++uv) {
+            if (code < 0) {
+                // a quadrant as it is: nothing to add, nothing to round
+                const int Q = -1 - code;
+                s[uv] = v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)];
+                unpack_elems<T>(s[uv], x[uv]);
+                continue;
+            }
             float acc[kEPT2];
 #pragma unroll
             for (int e = 0; e < kEPT2; ++e) acc[e] = 0.f;
 #pragma unroll
             for (int Q = 0; Q < 4; ++Q) {
-                const int cf = p.l1[q][Q];
+                const int cf = first_coef(SIDE, q, Q);
                 if (cf == 0) continue;
-                float x[kEPT2];
-                unpack_elems<T>(v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)], x);
+                float t[kEPT2];
+                unpack_elems<T>(v[(2 * (Q >> 1) + (uv >> 1)) * 4 + 2 * (Q & 1) + (uv & 1)], t);
 #pragma unroll
-                for (int e = 0; e < kEPT2; ++e) acc[e] = cf > 0 ? acc[e] + x[e] : acc[e] - x[e];
+                for (int e = 0; e < kEPT2; ++e) acc[e] = cf > 0 ? acc[e] + t[e] : acc[e] - t[e];
             }
-            s[uv] = pack_elems<T>(acc);   // exact for a single quadrant, the one rounding of a sum otherwise
-            const int dst = p.l1_sum[q];
-            if (dst >= 0 && ((p.keep >> uv) & 1))
-                store_hinted(s[uv], reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s1[dst]) + ((uv >> 1) * p.q1_u + (uv & 1) * p.q1_v + o1) * ES), p.streaming);
+            s[uv] = pack_elems<T>(acc);   // the one rounding of a first-level sum
+            unpack_elems<T>(s[uv], x[uv]);
+            if ((kept_quarters(SIDE, ALGO2) >> uv) & 1)
+                store_hinted(s[uv], reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s1[code]) + ((uv >> 1) * p.q1_u + (uv & 1) * p.q1_v + o1) * ES), p.streaming);
         }
-        float x[4][kEPT2];
 #pragma unroll
-        for (int uv = 0; uv < 4; ++uv) unpack_elems<T>(s[uv], x[uv]);
-        for (int o = 0; o < p.nout2; ++o) {
+        for (int o = 0; o < NOUT2; ++o) {
             float acc[kEPT2];
 #pragma unroll
             for (int e = 0; e < kEPT2; ++e) {
                 float a = 0.f;
 #pragma unroll
                 for (int uv = 0; uv < 4; ++uv) {
-                    const int cf = p.c2[o][uv];
+                    const int cf = second_coef(SIDE, ALGO2, o, uv);
                     if (cf > 0) a += x[uv][e]; else if (cf < 0) a -= x[uv][e];
                 }
                 acc[e] = a;
@@ -327,6 +403,16 @@ __global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) 
             store_hinted(pack_elems<T>(acc), reinterpret_cast<vec_t*>(reinterpret_cast<char*>(p.s2[q]) + (int64_t)o * p.s2_stride + o2), p.streaming);
         }
     }
+}
+
+template <class T>
+__global__ void __launch_bounds__(256) quad_combos2_kernel(const Combo2Pair pp) {
+    const Combo2Params& p = pp.side[blockIdx.z];
+    const int variant = __builtin_amdgcn_readfirstlane(2 * p.side + (p.algo2 == STHIP_STRASSEN ? 0 : 1));
+    if (variant == 0) combos2_body<T, 0, STHIP_STRASSEN>(p);
+    else if (variant == 1) combos2_body<T, 0, STHIP_WINOGRAD>(p);
+    else if (variant == 2) combos2_body<T, 1, STHIP_STRASSEN>(p);
+    else combos2_body<T, 1, STHIP_WINOGRAD>(p);
 }
 
 // Quadrant sums each algorithm needs, as coefficients over (X11, X12, X21, X22).
@@ -835,6 +921,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
                 cp.ld_out = side == 0 ? sa_ld : sb_ld;
                 cp.bs_out = (int64_t)((side == 0 ? sa_b : sb_b) / 2);
                 cp.nout = nout; cp.rows = (int)r_ext; cp.chunks_per_row = (int)(c_ext / 8);
+                cp.table = (algo == STHIP_STRASSEN ? 0 : 2) + side;
                 most = std::max(most, r_ext * (c_ext / 8));
             }
             dim3 grid((unsigned)ceil_div(most, 256), (unsigned)batch, (unsigned)sides);
@@ -1162,6 +1249,7 @@ static int64_t fill_combo(ComboParams& cp, View X, int64_t r_blk, int64_t c_blk,
     cp.ld_in = row_major ? X.rs : X.cs;
     cp.ld_out = cols;
     cp.nout = nout; cp.rows = (int)rows; cp.chunks_per_row = (int)(cols / epc);
+    cp.table = coef == kStrA ? 0 : coef == kStrB ? 1 : coef == kWinA ? 2 : coef == kWinB ? 3 : -1;
     return rows * (cols / epc);
 }
 
@@ -1216,27 +1304,12 @@ static int64_t fill_combo2(Combo2Params& cp, View X, int64_t rq, int64_t cq, cha
     const bool row_major = X.cs == 1;
     for (int R = 0; R < 4; ++R)
         for (int C = 0; C < 4; ++C) cp.x[4 * R + C] = X.p + ((int64_t)R * rq * X.rs + (int64_t)C * cq * X.cs) * es;
-    // first-level operands in kernel order (level_operands): A side A11 S9 S2 S7 S5 S3 A22 with the
-    // sums numbered as the outputs of kStrA (S2 S3 S5 S7 S9 = 0..4); B side S1 S10 B22 S8 S6 B11 S4
-    // (kStrB: S1 S4 S6 S8 S10 = 0..4)
-    static const signed char kFirstA[7] = {-1, 4, 0, 3, 2, 1, -4}, kFirstB[7] = {0, 4, -4, 3, 2, -1, 1};   // >= 0: sum; -1 - q: quadrant q
-    for (int p = 0; p < 7; ++p) {
-        const int f = side == 0 ? kFirstA[p] : kFirstB[p];
-        cp.l1_sum[p] = (signed char)(f >= 0 ? f : -1);
-        for (int Q = 0; Q < 4; ++Q)
-            cp.l1[p][Q] = f >= 0 ? (side == 0 ? kStrA[f][Q] : kStrB[f][Q]) : (Q == -1 - f ? 1 : 0);
-        cp.s2[p] = S2 + (size_t)p * 5 * s2_b;
-    }
+    // the kernel holds the coefficient tables of both levels (str_coef, first_code, ...): first level
+    // Strassen in the order of level_operands, second level `algo2`
+    for (int p = 0; p < 7; ++p) cp.s2[p] = S2 + (size_t)p * 5 * s2_b;
     for (int o = 0; o < 5; ++o) cp.s1[o] = S1 + (size_t)o * s1_b;
     cp.s2_stride = (int64_t)s2_b;
-    const bool strassen2 = algo2 == STHIP_STRASSEN;
-    cp.nout2 = strassen2 ? 5 : 4;
-    for (int o = 0; o < cp.nout2; ++o)
-        for (int uv = 0; uv < 4; ++uv)
-            cp.c2[o][uv] = strassen2 ? (side == 0 ? kStrA[o][uv] : kStrB[o][uv]) : (side == 0 ? kWinA[o][uv] : kWinB[o][uv]);
-    // quarters of a first-level sum that the second level multiplies as they are (level_operands):
-    // Strassen 11 and 22; Winograd 11, 12 and 22 of an A-side operand, 11, 21 and 22 of a B-side one
-    cp.keep = strassen2 ? 0x9 : (side == 0 ? 0xB : 0xD);
+    cp.side = side; cp.algo2 = algo2;
     const int64_t rows = row_major ? rq : cq, cols = row_major ? cq : rq;   // quarter block, storage order
     cp.ld_in = row_major ? X.rs : X.cs;
     cp.ld1 = 2 * cols;
