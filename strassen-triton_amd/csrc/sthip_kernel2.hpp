@@ -49,6 +49,8 @@ struct Gemm2Params {
     int out_f32, accumulate, group_m;
     int c_wide;           // 256 x 256 kernel: C, its rows and its product / batch strides are 16-byte aligned
     int c_stream;         // 256 x 256 kernel: store the result tiles with the streaming hint
+    int xcd_chunks;       // 256 x 256 kernel: products of fewer than 256 tiles go to the XCDs 32 tiles at a time (1-D grid)
+    int nbatch;           // batch entries, when xcd_chunks is set (the grid does not tell)
 };
 
 __device__ __forceinline__ void wait_vmcnt(int n) {

@@ -405,13 +405,38 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     // blockIdx.x = product * tiles + tile: the XCD-aware renumbering works within one product
     const int tiles = P.tiles_m * P.tiles_n;
-    const int prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
-    GemmParams tp;
-    tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = P.group_m;
-    int tm, tn;
-    tile_coords_in(tp, (int)blockIdx.x - prod * tiles, tiles, tm, tn);
+    int prod, batch, tm, tn;
+    const int nprod = P.nprod > 0 ? P.nprod : 1;
+    // Products of fewer than 256 tiles (several run at once): with the numbering above every XCD
+    // would hold eight tiles of each of four products.  Instead the grid is one-dimensional over
+    // (batch entry, product, tile) and XCD x (workgroups x, x + 8, ...) takes whole chunks of 32
+    // tiles -- four tile rows by eight columns of ONE product, which share their operand panels in
+    // that XCD's L2 -- chunk x first, then x + 8, ...  Chunks beyond the last full set of eight are
+    // numbered the plain way.
+    const int chunks = P.xcd_chunks ? (nprod * P.nbatch * tiles / 32) / 8 * 8 : 0;
+    const int bid = (int)blockIdx.x;
+    if (P.xcd_chunks && bid < chunks * 32) {
+        const int x = bid & 7, j = bid >> 3;
+        const int h = (j >> 5) * 8 + x, per = tiles / 32;
+        const int pb = h / per, part = h - pb * per, l = j & 31;
+        batch = pb / nprod; prod = pb - batch * nprod;
+        const int t = part * 32 + l;                 // tile of the product, walked four rows at a time
+        const int width = 4 * P.tiles_n, grp = t / width, in = t - grp * width;
+        tm = grp * 4 + (in & 3); tn = in >> 2;
+    } else {
+        int rest = bid - chunks * 32, first = chunks * 32 / tiles;   // whole products before `rest`
+        if (!P.xcd_chunks) { rest = bid; first = 0; }
+        const int pl = rest / tiles;
+        GemmParams tp;
+        tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = P.group_m;
+        tile_coords_in(tp, rest - pl * tiles, tiles, tm, tn);
+        const int pb = first + pl;
+        if (P.xcd_chunks) { batch = pb / nprod; prod = pb - batch * nprod; }
+        else { batch = blockIdx.y; prod = pb; }
+    }
+    prod = __builtin_amdgcn_readfirstlane(prod);
+    batch = __builtin_amdgcn_readfirstlane(batch);
     const int tile_m = tm * kBM4, tile_n = tn * kBN4;
-    const int batch = blockIdx.y;
     char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int KT = P.Kh / bk4<T>();

@@ -102,8 +102,16 @@ hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
     hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes4);
     if (e != hipSuccess) return e;
     const int nprod = p.nprod > 0 ? p.nprod : 1;
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n * nprod), (unsigned)batch, 1);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, p);
+    const int tiles = p.tiles_m * p.tiles_n;
+    Gemm2Params q = p;
+    // several small products at once: XCD-chunked numbering (see gemm4_kernel) on a one-dimensional grid
+    // (measured: grouped launch of config 4 1.585 -> 1.545 ms, two-level 8192^3 0.787 -> 0.766 ms)
+    q.xcd_chunks = (tiles == 32 || tiles == 64 || tiles == 128) && p.tiles_m % 4 == 0 && nprod * batch * tiles >= 256 &&
+                   (int64_t)nprod * batch * tiles < (1 << 30) ? 1 : 0;
+    q.nbatch = batch;
+    dim3 grid((unsigned)(tiles * nprod), (unsigned)batch, 1);
+    if (q.xcd_chunks) grid = dim3((unsigned)(tiles * nprod * batch), 1, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(kThreads4), kSmemBytes4, stream, q);
     return hipGetLastError();
 }
 
