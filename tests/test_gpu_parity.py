@@ -430,6 +430,32 @@ def test_large_tile_store_alignment(hip, force_tile, dtype, pad, off, algo, leve
     assert torch.all(buf[:, :off] == 7) and torch.all(buf[:, off + N:] == 7)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("algo,levels,shape,batch", [
+    ("classic", 0, (2048, 2048, 128), 5),      # 64 tiles per product: ten chunks of 32, eight dealt to the XCDs, two numbered plainly
+    ("classic", 0, (1024, 2048, 128), 9),      # 32 tiles per product, nine products
+    ("classic", 0, (2048, 4096, 128), 3),      # 128 tiles per product
+    ("strassen", 1, (2048, 4096, 2048), 2),    # seven products of 32 tiles, two batch entries
+    ("strassen", 1, (4096, 4096, 2048), 1),    # seven products of 64 tiles: 448 = 256 chunked + 192 plain
+    ("winograd", 1, (4096, 8192, 2048), 1),    # seven products of 128 tiles
+    ("strassen", 2, (8192, 8192, 4096), 1),    # 49 products of 64 tiles
+])
+def test_large_tile_small_products_cover_every_tile(hip, force_tile, dtype, algo, levels, shape, batch):
+    """Products of fewer than 256 tiles are dealt to the XCDs in chunks of 32 tiles on a
+    one-dimensional grid over (batch entry, product, tile).  Every tile of every product must be
+    computed exactly once: the result buffer starts out filled with a sentinel, inputs are small
+    integers, and the output must be exact everywhere."""
+    force_tile("256x256")
+    M, N, K = shape
+    bs = (batch,) if batch > 1 else ()
+    A, B = _ints(bs + (M, K), 81, -1, 1, dtype), _ints(bs + (K, N), 82, -1, 1, dtype)
+    if dtype != torch.float32:
+        A[..., 128:] = 0   # |C| <= 128 stays exact in 16 bits at any k
+    out = torch.full(bs + (M, N), 777.0, dtype=dtype, device="cuda")
+    hip.gemm(A.cuda(), B.cuda(), out=out, algo=algo, levels=levels)
+    assert torch.equal(out.cpu().double(), A.double() @ B.double())
+
+
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("algo,levels,shape,batch", [
     ("classic", 0, (4096, 4096, 96), 1),       # 256 tiles of 256 x 256
