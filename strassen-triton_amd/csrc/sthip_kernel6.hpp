@@ -227,8 +227,13 @@ __global__ void __launch_bounds__(kThreads6) gemm6_kernel(const Gemm6Params P) {
     __shared__ __attribute__((aligned(1024))) char smem[2 * kStageBytes6];
     const int tiles = P.tiles_m * P.tiles_n;
     const int prod = __builtin_amdgcn_readfirstlane((int)blockIdx.x / tiles);
-    const int t = (int)blockIdx.x - prod * tiles;
-    const int tile_m = (t / P.tiles_n) * kBM6, tile_n = (t % P.tiles_n) * kBN6;
+    // XCD-aware walk within the product (tile_coords_in): each XCD owns a contiguous run of tiles, taken
+    // eight tile rows at a time, so that neighbours share operand panels in that XCD's L2
+    GemmParams tp;
+    tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = 8;
+    int tm, tn;
+    tile_coords_in(tp, (int)blockIdx.x - prod * tiles, tiles, tm, tn);
+    const int tile_m = tm * kBM6, tile_n = tn * kBN6;
     const bool a_sum = P.a[prod].sign != 0, b_sum = P.b[prod].sign != 0;
     if (a_sum && b_sum) run6<B_KC, true, true>(P, smem, prod, tile_m, tile_n);
     else if (a_sum) run6<B_KC, true, false>(P, smem, prod, tile_m, tile_n);
