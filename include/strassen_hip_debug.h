@@ -19,8 +19,9 @@ int sthip_debug_transpose_read(void* out, void* stream);
  * bit 1 = grouped GEMM, bit 2 = recombination pass; bit 3 lets two-level calls run as one
  * 49-product launch instead of the host recursion; bit 4 runs large one-level 16-bit Strassen
  * calls as ONE launch whose workgroups are the sums, the product tiles and the recombination --
- * same bits, slower than the three launches on MI355X, hence off by default; default 15) and
- * returns the previous mask.
+ * same bits, slower than the three launches on MI355X, hence off by default; bit 5 makes the
+ * 256 x 256 kernel launch one workgroup per tile instead of one per CU that walks the tiles --
+ * same bits, slower; default 15) and returns the previous mask.
  * With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so the
  * dominant kernel can be timed alone. */
 int sthip_debug_set_stages(int mask);

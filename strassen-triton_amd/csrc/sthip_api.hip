@@ -22,7 +22,7 @@ static thread_local char g_err[512] = "";
 // Stages of the pipelined path that run: bit 0 = quadrant-sum pre-pass, bit 1 = grouped GEMM,
 // bit 2 = recombination pass, bit 3 = two levels may run as one 49-product launch, bit 4 = one level
 // may run as ONE launch (sums, products and recombination as work items of one grid).
-constexpr int kAllStages = 31;
+constexpr int kAllStages = 63;
 constexpr int kDefaultStages = 15;   // the one-launch form is slower than the three launches (sthip_kernel5.hpp): off unless asked for
 static std::atomic<int> g_debug_stages{kDefaultStages};
 // Forced tile: 0 = the tile table decides, 2 = 128 x 128, 3 = 256 x 128, 4 = 256 x 256, 5 = 128 x 128 with
@@ -970,6 +970,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
                 p.tiles_m = (int)(Mh / kBM4); p.tiles_n = (int)(Nh / kBN4);
                 p.group_m = 4;
                 p.c_wide = wide_rows(p.C, p.c_rs, p.c_ps, p.c_bs);
+                p.one_tile_per_wg = (cx.stages & 32) ? 1 : 0;
                 e = t4->fn[b_kc ? 1 : 0](p, (int)batch, cx.stream);
             } else {
                 const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);
@@ -1000,6 +1001,7 @@ static int launch_pipelined(View A, View B, char* C, int64_t c_rs, int64_t batch
         p.group_m = 4; p.nprod = 1;
         p.c_stream = 1;   // the final result: not read again by this call
         p.c_wide = wide_rows(p.C, p.c_rs, 0, p.c_bs);
+        p.one_tile_per_wg = (cx.stages & 32) ? 1 : 0;
         e = t4->fn[b_kc ? 1 : 0](p, (int)batch, cx.stream);
     } else if (pick == 3) {
         p.tiles_m = (int)(Mh / kBM3);
@@ -1392,6 +1394,7 @@ static int two_level_flat(View A, View B, char* C, int64_t c_rs, int64_t mh, int
     } else if (big) {
         g.tiles_m = (int)(mq / kBM4); g.tiles_n = (int)(nq / kBN4);
         g.c_wide = wide_rows(g.C, g.c_rs, g.c_ps, 0);
+        g.one_tile_per_wg = (cx.stages & 32) ? 1 : 0;
         e = t4->fn[b_kc ? 1 : 0](g, 1, cx.stream);
     } else {
         const LaunchTable2* t = table2_for(dt, STHIP_CLASSIC);

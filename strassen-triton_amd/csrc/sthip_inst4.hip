@@ -14,6 +14,8 @@ typedef bf16_t InstT;
 
 template __global__ void gemm4_kernel<InstT, false>(const Gemm2Params);
 template __global__ void gemm4_kernel<InstT, true>(const Gemm2Params);
+template __global__ void gemm4p_kernel<InstT, false>(const Gemm2Params);
+template __global__ void gemm4p_kernel<InstT, true>(const Gemm2Params);
 
 #ifndef __HIP_DEVICE_COMPILE__
 #define STHIP_CAT2(a, b) kLaunch4_##a

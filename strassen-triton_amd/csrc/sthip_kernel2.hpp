@@ -50,7 +50,8 @@ struct Gemm2Params {
     int c_wide;           // 256 x 256 kernel: C, its rows and its product / batch strides are 16-byte aligned
     int c_stream;         // 256 x 256 kernel: store the result tiles with the streaming hint
     int xcd_chunks;       // 256 x 256 kernel: products of fewer than 256 tiles go to the XCDs 32 tiles at a time (1-D grid)
-    int nbatch;           // batch entries, when xcd_chunks is set (the grid does not tell)
+    int nbatch;           // 256 x 256 kernel: batch entries (its grid is one-dimensional over batch entry, product and tile)
+    int one_tile_per_wg;  // 256 x 256 kernel: never let a workgroup walk several tiles (test and timing switch)
 };
 
 __device__ __forceinline__ void wait_vmcnt(int n) {

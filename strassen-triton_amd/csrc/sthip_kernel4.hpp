@@ -45,6 +45,47 @@ constexpr int kATile4 = kBM4 * kBK4 * 2;                 // 32 KiB
 constexpr int kBTile4 = kBN4 * kBK4 * 2;                 // 32 KiB
 constexpr int kStageBytes4 = kATile4 + kBTile4;          // 64 KiB
 constexpr int kSmemBytes4 = kStages4 * kStageBytes4;     // 128 KiB
+constexpr int kOutStage4 = 4096;                         // per wave: 32 rows x 128 bytes of a 16-bit result on their way out
+constexpr int kSmemBytes4p = kSmemBytes4 + 8 * kOutStage4;   // 160 KiB: the stage buffers stay in use while a tile is stored
+
+// Tile `id` of a launch, numbered over (batch entry, product, tile of the product).
+// Products of at least 256 tiles: the XCD-aware renumbering works within one product (workgroup x,
+// x + 8, ... run on XCD x; ids are renumbered so that an XCD owns a contiguous run of tiles).
+// Products of fewer than 256 tiles (several run at once): that numbering would give every XCD eight
+// tiles of each of four products.  Instead XCD x takes whole chunks of 32 tiles -- four tile rows
+// by eight columns of ONE product, which share their operand panels in that XCD's L2 -- chunk x
+// first, then x + 8, ...  Chunks beyond the last full set of eight are numbered the plain way.
+__device__ __forceinline__ void map_tile4(const Gemm2Params& P, int id, int& prod, int& batch, int& tm, int& tn) {
+    // `z` is zero, but not to the compiler: everything below is then computed where it is needed, once
+    // per tile.  Otherwise the dozen values that are the same for every tile are kept in scalar
+    // registers across the main loop, which then spills.
+    int z = 0;
+    asm volatile("" : "+s"(z));
+    const int tiles_m = P.tiles_m + z, tiles_n = P.tiles_n + z, tiles = tiles_m * tiles_n;
+    const int nprod = (P.nprod > 0 ? P.nprod : 1) + z;
+    const int chunks = P.xcd_chunks + z ? (nprod * P.nbatch * tiles / 32) / 8 * 8 : 0;
+    int pb;
+    if (id < chunks * 32) {
+        const int x = id & 7, j = id >> 3;
+        const int h = (j >> 5) * 8 + x, per = tiles / 32;
+        pb = h / per;
+        const int part = h - pb * per, l = j & 31;
+        const int t = part * 32 + l;                 // tile of the product, walked four rows at a time
+        const int width = 4 * tiles_n, grp = t / width, in = t - grp * width;
+        tm = grp * 4 + (in & 3); tn = in >> 2;
+    } else {
+        const int rest = id - chunks * 32, first = chunks * 32 / tiles;   // whole products before `rest`
+        const int pl = rest / tiles;
+        GemmParams tp;
+        tp.tiles_m = tiles_m; tp.tiles_n = tiles_n; tp.group_m = P.group_m + z;
+        tile_coords_in(tp, rest - pl * tiles, tiles, tm, tn);
+        pb = first + pl;
+    }
+    batch = __builtin_amdgcn_readfirstlane(pb / nprod);
+    prod = __builtin_amdgcn_readfirstlane(pb - batch * nprod);
+    tm = __builtin_amdgcn_readfirstlane(tm);   // uniform by construction; the loader needs its bases in scalar registers
+    tn = __builtin_amdgcn_readfirstlane(tn);
+}
 
 // A and k-contiguous B: 256 rows x 8 chunks; wave w loads rows 32 w + 8 i + L/8, i = 0..3,
 // chunk (L%8) ^ ((row/2)%8).  n-contiguous B: 64 k-rows x 32 chunks (512 bytes); wave w loads
@@ -60,6 +101,7 @@ struct Loader4 {
     uint32_t a_voff[2], b_voff[2];   // index i % 2 of the wave's load i
     int seg, kt, total_seg, KT;
     int batch, tile_m, tile_n, wave;
+    int id, stride, total_ids;   // stride > 0: after the KT steps of tile `id` the loader goes on with tile id + stride
     const Gemm2Params* P;
 
     __device__ __forceinline__ void point_at_segment() {
@@ -121,7 +163,16 @@ struct Loader4 {
         b_base += b_step_bytes;
         if (++kt == KT) {
             kt = 0;
-            if (++seg < total_seg) point_at_segment();
+            if (stride > 0) {
+                id += stride;
+                if (id < total_ids) {
+                    int tm, tn;
+                    map_tile4(*P, id, seg, batch, tm, tn);
+                    tile_m = tm * kBM4; tile_n = tn * kBN4;
+                    total_seg = seg + 1;
+                    point_at_segment();
+                } else seg = total_seg;
+            } else if (++seg < total_seg) point_at_segment();
         }
     }
 
@@ -290,10 +341,20 @@ struct Pipe4 {
     }
 };
 
+// The lane index as a value the compiler cannot see through: everything a store routine derives from
+// it is then computed where the routine runs.  (Otherwise the per-lane addresses of the stores, being
+// the same for every tile a workgroup computes, are hoisted out of the tile loop and held in registers
+// across the main loop, which has none to spare: eight spills per k-step.)
+__device__ __forceinline__ int opaque_lane4() {
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
+
 // Lane l of MFMA tile (i, j) holds m = 16 i + l % 16 and n = 16 j + 4 (l / 16) + 0..3.
 template <class T>
 __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& P, char* Cb, int quad, int row, int col) {
-    const int lane = threadIdx.x & 63;
+    const int lane = opaque_lane4();
     const int esz = P.out_f32 ? 4 : 2;
     const int m0 = (quad >> 1) * P.Mh + row + (lane & 15);
     const int n0 = (quad & 1) * P.Nh + col + 4 * (lane >> 4);
@@ -342,7 +403,7 @@ __device__ __forceinline__ void store_tile4(const Acc4& acc, const Gemm2Params& 
 template <class T>
 __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Params& P, char* Cb, char* smem,
                                                 int wave, int row, int col) {
-    const int lane = threadIdx.x & 63;
+    const int lane = opaque_lane4();
     const int l16 = lane & 15, q = lane >> 4;
     char* w = smem + wave * 16384;
     uint32_t waddr[4];
@@ -379,7 +440,7 @@ __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Para
 // Every store instruction then writes four rows x 256 contiguous bytes.
 __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2Params& P, char* Cb, char* smem,
                                                     int wave, int row, int col) {
-    const int lane = threadIdx.x & 63;
+    const int lane = opaque_lane4();
     const int l16 = lane & 15, q = lane >> 4;
     char* w = smem + wave * 16384;
     float* dst = reinterpret_cast<float*>(Cb) + (int64_t)(row + q) * P.c_rs + (col + 4 * l16);
@@ -400,60 +461,77 @@ __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2
     }
 }
 
-template <class T, bool B_KC>
-__global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
-    extern __shared__ __attribute__((aligned(1024))) char smem[];
-    // blockIdx.x = product * tiles + tile: the XCD-aware renumbering works within one product
-    const int tiles = P.tiles_m * P.tiles_n;
-    int prod, batch, tm, tn;
-    const int nprod = P.nprod > 0 ? P.nprod : 1;
-    // Products of fewer than 256 tiles (several run at once): with the numbering above every XCD
-    // would hold eight tiles of each of four products.  Instead the grid is one-dimensional over
-    // (batch entry, product, tile) and XCD x (workgroups x, x + 8, ...) takes whole chunks of 32
-    // tiles -- four tile rows by eight columns of ONE product, which share their operand panels in
-    // that XCD's L2 -- chunk x first, then x + 8, ...  Chunks beyond the last full set of eight are
-    // numbered the plain way.
-    const int chunks = P.xcd_chunks ? (nprod * P.nbatch * tiles / 32) / 8 * 8 : 0;
-    const int bid = (int)blockIdx.x;
-    if (P.xcd_chunks && bid < chunks * 32) {
-        const int x = bid & 7, j = bid >> 3;
-        const int h = (j >> 5) * 8 + x, per = tiles / 32;
-        const int pb = h / per, part = h - pb * per, l = j & 31;
-        batch = pb / nprod; prod = pb - batch * nprod;
-        const int t = part * 32 + l;                 // tile of the product, walked four rows at a time
-        const int width = 4 * P.tiles_n, grp = t / width, in = t - grp * width;
-        tm = grp * 4 + (in & 3); tn = in >> 2;
-    } else {
-        int rest = bid - chunks * 32, first = chunks * 32 / tiles;   // whole products before `rest`
-        if (!P.xcd_chunks) { rest = bid; first = 0; }
-        const int pl = rest / tiles;
-        GemmParams tp;
-        tp.tiles_m = P.tiles_m; tp.tiles_n = P.tiles_n; tp.group_m = P.group_m;
-        tile_coords_in(tp, rest - pl * tiles, tiles, tm, tn);
-        const int pb = first + pl;
-        if (P.xcd_chunks) { batch = pb / nprod; prod = pb - batch * nprod; }
-        else { batch = blockIdx.y; prod = pb; }
+// The same 16-bit store for a workgroup that goes on to another tile: the stage buffers already
+// hold (or are receiving) the next tile's first k-steps, so each wave stages its 128 x 64 tile in
+// four passes of 32 rows through 4 KiB of its own beyond the stage buffers.  Row r of a pass at
+// r * 128, the 8-byte chunk c of a row at (c ^ 2 ((r / 2) % 8)) * 8 as above; the wave reads back
+// what it wrote itself (LDS keeps a wave's accesses in order), so no barrier is involved.
+template <class T>
+__device__ __forceinline__ void store_tile4_own(const Acc4& acc, const Gemm2Params& P, char* Cb, char* out_stage,
+                                                int wave, int row, int col) {
+    const int lane = opaque_lane4();
+    const int l16 = lane & 15, q = lane >> 4;
+    char* w = out_stage + wave * kOutStage4;
+    uint32_t waddr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) waddr[j] = l16 * 128 + (((4 * j + q) ^ (2 * (l16 >> 1))) * 8);
+    const int r8 = lane >> 3, c16 = lane & 7;
+    char* dst = Cb + ((int64_t)(row + r8) * P.c_rs + (col + 8 * c16)) * 2;
+    const int64_t step = (int64_t)8 * P.c_rs * 2;
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) {
+            const int i = 2 * h + ii;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                u32x2 o;
+                if constexpr (__is_same(T, bf16_t)) { o[0] = pack_bf16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_bf16(acc.t[i][j][2], acc.t[i][j][3]); }
+                else { o[0] = pack_f16(acc.t[i][j][0], acc.t[i][j][1]); o[1] = pack_f16(acc.t[i][j][2], acc.t[i][j][3]); }
+                *reinterpret_cast<u32x2*>(w + ii * 2048 + waddr[j]) = o;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int rr = ((8 * r + r8) >> 1) & 7;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(w + (8 * r + r8) * 128 + ((c16 ^ rr) * 16));
+            store_hinted(v, reinterpret_cast<u32x4*>(dst + (4 * h + r) * step), P.c_stream);
+        }
     }
-    prod = __builtin_amdgcn_readfirstlane(prod);
-    batch = __builtin_amdgcn_readfirstlane(batch);
-    const int tile_m = tm * kBM4, tile_n = tn * kBN4;
-    char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int KT = P.Kh / bk4<T>();
+}
 
-    Pipe4<T, B_KC> pipe;
+// Set-up shared by the two kernels below: the pipeline of workgroup blockIdx.x, pointed at its first tile.
+template <class T, bool B_KC>
+__device__ __forceinline__ void begin4(Pipe4<T, B_KC>& pipe, const Gemm2Params& P, char* smem, int wave, int KT,
+                                       int id, int stride, int total, int& prod, int& batch, int& tm, int& tn) {
+    map_tile4(P, id, prod, batch, tm, tn);
     pipe.smem = smem;
     pipe.smem_addr = (uint32_t)(uintptr_t)(lptr_t)smem;
     pipe.wm = (wave >> 2) * 128;
     pipe.wn = (wave & 3) * 64;
-    pipe.total = KT;
+    pipe.total = KT * ((total - 1 - id) / stride + 1);
     pipe.ld.P = &P;
     pipe.ld.wave = wave;
     pipe.ld.seg = prod; pipe.ld.kt = 0; pipe.ld.total_seg = prod + 1; pipe.ld.KT = KT;
-    pipe.ld.batch = batch; pipe.ld.tile_m = tile_m; pipe.ld.tile_n = tile_n;
+    pipe.ld.batch = batch; pipe.ld.tile_m = tm * kBM4; pipe.ld.tile_n = tn * kBN4;
+    pipe.ld.id = id; pipe.ld.stride = stride; pipe.ld.total_ids = total;
     pipe.ld.point_at_segment();
     pipe.start();
+}
 
+// One tile per workgroup (blockIdx.x = tile id, see map_tile4), any kind of result.
+template <class T, bool B_KC>
+__global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int total = P.tiles_m * P.tiles_n * (P.nprod > 0 ? P.nprod : 1) * P.nbatch;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int KT = P.Kh / bk4<T>();
+    const int id = __builtin_amdgcn_readfirstlane((int)blockIdx.x);
+    int prod, batch, tm, tn;
+    Pipe4<T, B_KC> pipe;
+    begin4<T, B_KC>(pipe, P, smem, wave, KT, id, total, total, prod, batch, tm, tn);
+    const int tile_m = tm * kBM4, tile_n = tn * kBN4;
+    char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * (P.out_f32 ? 4 : 2);
     Acc4 r;
     r.zero();
     pipe.run(r, KT);
@@ -465,6 +543,49 @@ __global__ void __launch_bounds__(kThreads4) gemm4_kernel(const Gemm2Params P) {
         store_tile4_lds_f32(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
     } else {
         store_tile4<T>(r, P, Cb, 0, tile_m + pipe.wm, tile_n + pipe.wn);
+    }
+}
+
+// Fewer workgroups than tiles (one per CU): workgroup b computes tiles b, b + gridDim.x, ... as ONE
+// software pipeline.  The loader runs on into the next tile, whose first k-steps are in flight
+// while this tile's last ones are multiplied and while its result is stored, so that a tile costs
+// its k-steps and a store, not a dispatch, a prologue and a drain as well.  16-bit results with
+// 16-byte aligned rows, not accumulating (the launcher sees to it).
+template <class T, bool B_KC>
+__global__ void __launch_bounds__(kThreads4) gemm4p_kernel(const Gemm2Params P) {
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int total = P.tiles_m * P.tiles_n * (P.nprod > 0 ? P.nprod : 1) * P.nbatch;
+    const int stride = (int)gridDim.x;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int KT = P.Kh / bk4<T>();
+    int id = __builtin_amdgcn_readfirstlane((int)blockIdx.x);
+    int prod, batch, tm, tn;
+    Pipe4<T, B_KC> pipe;
+    begin4<T, B_KC>(pipe, P, smem, wave, KT, id, stride, total, prod, batch, tm, tn);
+    for (;;) {
+        const int tile_m = tm * kBM4, tile_n = tn * kBN4;
+        char* Cb = reinterpret_cast<char*>(P.C) + ((int64_t)batch * P.c_bs + (int64_t)prod * P.c_ps) * 2;
+        Acc4 r;
+        r.zero();
+        pipe.run(r, KT);
+        if (id + stride >= total) {
+            __syncthreads();   // every wave has read its last fragments: the stage buffers are free
+            store_tile4_lds<T>(r, P, Cb, smem, wave, tile_m + pipe.wm, tile_n + pipe.wn);
+            break;
+        }
+        store_tile4_own<T>(r, P, Cb, smem + kSmemBytes4, wave, tile_m + pipe.wm, tile_n + pipe.wn);
+        id += stride;
+        map_tile4(P, id, prod, batch, tm, tn);
+        // The first fragments of the next tile were read before the store; reading them again here
+        // means they need not stay in registers across the store.
+        pipe.read_frags(0, pipe.slot, 0);
+        // Nothing the compiler knows of may be outstanding when the main loop starts again: it guards
+        // the data registers of the stores above until they have completed, with vmcnt waits INSIDE
+        // the loop, where a wait also counts the direct-to-LDS loads it does not know of and drains
+        // them at every k-step (measured: +20 %).  The empty statements keep the stores before the wait.
+        asm volatile("" ::: "memory");
+        wait_vmcnt_imm<0>();
+        asm volatile("" ::: "memory");
     }
 }
 

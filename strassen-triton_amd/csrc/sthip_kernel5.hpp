@@ -280,6 +280,7 @@ __global__ void __launch_bounds__(kThreads4) fused5_kernel(const Fused5Params P)
     pipe.ld.wave = wave;
     pipe.ld.seg = prod; pipe.ld.kt = 0; pipe.ld.total_seg = prod + 1; pipe.ld.KT = KT;
     pipe.ld.batch = 0; pipe.ld.tile_m = tile_m; pipe.ld.tile_n = tile_n;
+    pipe.ld.stride = 0; pipe.ld.id = 0; pipe.ld.total_ids = 0;
     pipe.ld.point_at_segment();
     pipe.start();
 

@@ -516,6 +516,41 @@ def test_fp32_two_levels_flat_against_host_recursion(hip, tb):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("algo,levels,shape,batch", [
+    ("classic", 0, (4352, 4096, 192), 1),      # 272 tiles: sixteen workgroups walk two tiles, the others one
+    ("classic", 0, (2048, 2048, 128), 9),      # 576 tiles over nine batch entries, dealt in chunks of 32
+    ("strassen", 1, (4096, 4096, 512), 1),     # 448 tiles in seven products
+    ("winograd", 1, (8192, 8192, 256), 1),     # 1792 tiles: seven per workgroup
+    ("strassen", 2, (8192, 8192, 512), 1),     # 3136 tiles in 49 products
+])
+def test_workgroups_that_walk_tiles_same_bits(hip, force_tile, dtype, tb, algo, levels, shape, batch):
+    """With more 256 x 256 tiles than CUs the large-tile kernel launches one workgroup per CU, which
+    walks its tiles as one software pipeline (the next tile's first k-steps load while this one is
+    stored).  Bit 5 of the debug stage mask switches back to one workgroup per tile: same arithmetic
+    in the same order, so the same bits; and both are exact on small integers."""
+    from strassen_hip import _capi
+    lib = _capi.load()
+    force_tile("256x256")
+    M, N, K = shape
+    bs = (batch,) if batch > 1 else ()
+    A, B = _gauss(bs + (M, K), 211, K ** -0.5, dtype).cuda(), _layout(_gauss(bs + (K, N), 212, 1.0, dtype), tb)
+    Ai, Bi = _ints(bs + (M, K), 213, -1, 1, dtype), _ints(bs + (K, N), 214, -1, 1, dtype)
+    Ai[..., 128:] = 0   # |C| <= 128 stays exact in 16 bits
+    out = torch.full(bs + (M, N), 777.0, dtype=dtype, device="cuda")
+    got = hip.gemm(A, B, algo=algo, levels=levels)
+    exact = hip.gemm(Ai.cuda(), _layout(Bi, tb), out=out, algo=algo, levels=levels)
+    prev = lib.sthip_debug_set_stages(15 | 32)
+    try:
+        want = hip.gemm(A, B, algo=algo, levels=levels)
+        torch.cuda.synchronize()
+    finally:
+        lib.sthip_debug_set_stages(prev)
+    assert torch.equal(got, want)
+    assert torch.equal(exact.cpu().double(), Ai.double() @ Bi.double())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape,tb", [((4096, 4096, 4096), False), ((4096, 4096, 4096), True), ((4096, 8192, 2048), True),
                                       ((4096, 6144, 4096), False)])
 def test_one_level_as_one_launch_same_bits(hip, dtype, shape, tb):
