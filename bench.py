@@ -156,7 +156,7 @@ def cpu_baseline(A, B, levels, dtype, algo):
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel, as measured with rocprofv3 --pmc FETCH_SIZE /
     WRITE_SIZE and recorded in profiles/ (None if no such summary is committed)."""
-    rel = os.path.join("profiles", f"gemm_kernel_{workload}_hbm_traffic.txt")
+    rel = os.path.join("profiles", f"gemm4p_kernel_{workload}_hbm_traffic.txt")
     try:
         m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(os.path.join(ROOT, rel)).read(), re.M)
         return (float(m.group(1)), rel) if m else (None, None)
