@@ -144,57 +144,70 @@ __device__ __forceinline__ void run6(const Gemm6Params& P, char* smem, int prod,
         for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int l16 = lane & 15, g = lane >> 4;
-    auto compute = [&](int buf) {
+    // Fragments of one group of 16 k: component c is the element at k = 16 kg + 4 g + c of this lane's
+    // row / column.
+    struct Frag6 { f32x4 a[2], b[2]; };
+    auto read_frags = [&](Frag6& f, int buf, int kg) {
         const char* s = smem + buf * kStageBytes6;
 #pragma unroll
-        for (int kg = 0; kg < 2; ++kg) {
-            // component c of a fragment is the element at k = 16 kg + 4 g + c of this lane's row / column
-            f32x4 fa[2], fb[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int r = wm + 16 * i + l16;
-                fa[i] = *reinterpret_cast<const f32x4*>(s + r * 128 + (((kg * 4 + g) ^ ((r >> 1) & 7)) << 4));
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int n = wn + 16 * j + l16;
-                if constexpr (B_KC) {
-                    fb[j] = *reinterpret_cast<const f32x4*>(s + kTileBytes6 + n * 128 + (((kg * 4 + g) ^ ((n >> 1) & 7)) << 4));
-                } else {
-                    const char* p = s + kTileBytes6 + (kg * 16 + g * 4) * 256 + (((n >> 2) ^ (g << 2)) << 4) + (n & 3) * 4;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) fb[j][c] = *reinterpret_cast<const float*>(p + c * 256);
-                }
-            }
-            // operands swapped (rows of the instruction = n): a lane ends up with four consecutive n of one m
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-#pragma unroll
-                for (int i = 0; i < 2; ++i)
-#pragma unroll
-                    for (int j = 0; j < 2; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[j][c], fa[i][c], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 2; ++i) {
+            const int r = wm + 16 * i + l16;
+            f.a[i] = *reinterpret_cast<const f32x4*>(s + r * 128 + (((kg * 4 + g) ^ ((r >> 1) & 7)) << 4));
         }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = wn + 16 * j + l16;
+            if constexpr (B_KC) {
+                f.b[j] = *reinterpret_cast<const f32x4*>(s + kTileBytes6 + n * 128 + (((kg * 4 + g) ^ ((n >> 1) & 7)) << 4));
+            } else {
+                const char* p = s + kTileBytes6 + (kg * 16 + g * 4) * 256 + (((n >> 2) ^ (g << 2)) << 4) + (n & 3) * 4;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) f.b[j][c] = *reinterpret_cast<const float*>(p + c * 256);
+            }
+        }
+    };
+    // operands swapped (rows of the instruction = n): a lane ends up with four consecutive n of one m
+    auto multiply = [&](const Frag6& f) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.b[j][c], f.a[i][c], acc[i][j], 0, 0, 0);
     };
 
     // KT is even (host-checked): set 0 carries the even steps, set 1 the odd ones, one LDS buffer each.
-    // The loads of the steps two ahead are unconditional (the last iteration loads the last two steps
+    // One barrier per k-step, in its middle: while the first half of step g is multiplied its second
+    // half's fragments are read and step g + 1 goes from registers to the other LDS buffer; after the
+    // barrier the first fragments of step g + 1 are read while the second half of step g is
+    // multiplied, so that no fragment read is waited for with nothing to do.  (With the barrier
+    // between the steps the wait for the first fragments after it was exposed: 27.8 -> 26.5 us at 1024^3.)
+    // The loads of the steps two ahead are unconditional (the last iterations load the last two steps
     // again, unused), so that the number of loads in flight is the same at every wait.  (Two k-steps per
     // barrier on four LDS buffers were measured too: no faster at 1024^3, 8 % slower at 2048^3, where
     // 64 KiB of LDS per workgroup leaves fewer workgroups per CU.)
+    Frag6 f0, f1;
     fetch(0, 0);
     fetch(1, 1);
+    landed(0);
+    stage(0, 0);
+    fetch(0, min(2, KT - 2));
+    __syncthreads();
+    read_frags(f0, 0, 0);
+    auto half_steps = [&](int buf, int next_set, int next_step) {
+        read_frags(f1, buf, 1);
+        multiply(f0);
+        landed(next_set);
+        stage(next_set, buf ^ 1);
+        fetch(next_set, next_step);
+        __syncthreads();
+        read_frags(f0, buf ^ 1, 0);
+        multiply(f1);
+    };
     for (int kt = 0; kt < KT; kt += 2) {
-        landed(0);
-        stage(0, 0);
-        fetch(0, min(kt + 2, KT - 2));
-        __syncthreads();
-        compute(0);
-        landed(1);
-        stage(1, 1);
-        fetch(1, min(kt + 3, KT - 1));
-        __syncthreads();
-        compute(1);
+        half_steps(0, 1, min(kt + 3, KT - 1));
+        half_steps(1, 0, min(kt + 4, KT - 2));
     }
     // The reloads of the last two steps are still in flight.  Their target registers are dead to the
     // compiler, which would hand them to the epilogue (addresses, results) while the loads can still
