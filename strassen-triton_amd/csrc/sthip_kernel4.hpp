@@ -94,11 +94,26 @@ __device__ __forceinline__ void map_tile4(const Gemm2Params& P, int id, int& pro
 // n-contiguous fp32 B tile is 32 k-rows x 1024 bytes, one row per load: wave w loads k-rows
 // 4 w + i (i = 0..3), and slot s of row k holds chunk s ^ (((k / 4) % 4) * 4), so that the four k-rows a
 // fragment read touches (k = 4 g + c, lane group g) fall into different 64-byte bank groups.
+// lds_dma16 with the LDS address given as a uniform register plus a constant: one scalar instruction
+// for m0 and none for the global address (the rows of the load are part of the lane offset).
+__device__ __forceinline__ void lds_dma16_k(const void* sbase, uint32_t voff, uint32_t lds_addr, int k) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k) : "memory", "scc");
+}
+
+// 16-bit operands: the lane offset of load i includes the rows of load i (a_voff[i], b_voff[i]), so that
+// issuing a load in the main loop is three instructions (m0, a wait state, the load) and no scalar address
+// arithmetic: a wave issues in order, and a dozen scalar instructions and a branch per load held back the
+// matrix instructions behind them (measured: k-step 2890 -> 2750 cycles together with the row order of
+// Pipe4::run).  Lane offsets are 32-bit: 32 rows of the operand must span less than 4 GiB (the launcher
+// checks).  fp32 operands keep one offset per load parity and add the rows to the base: that kernel has no
+// registers to spare.
 template <int ES, bool B_KC>
 struct Loader4 {
+    static constexpr bool kRowsInLane = ES == 2;
     const char* a_base; const char* b_base;
     int64_t a_row_bytes, b_row_bytes, a_step_bytes, b_step_bytes;
-    uint32_t a_voff[2], b_voff[2];   // index i % 2 of the wave's load i
+    uint32_t a_voff[kRowsInLane ? 4 : 2], b_voff[kRowsInLane ? 4 : 2];   // load i of the wave (fp32: i % 2)
     int seg, kt, total_seg, KT;
     int batch, tile_m, tile_n, wave;
     int id, stride, total_ids;   // stride > 0: after the KT steps of tile `id` the loader goes on with tile id + stride
@@ -113,14 +128,26 @@ struct Loader4 {
         a_base = a + (int64_t)(tile_m + wave * 32) * s.a_ld * ES;
         a_row_bytes = 8 * s.a_ld * ES;
         a_step_bytes = kRowBytes4;
-        a_voff[0] = (uint32_t)((lane >> 3) * s.a_ld * ES + chunk0 * 16);
-        a_voff[1] = (uint32_t)((lane >> 3) * s.a_ld * ES + (chunk0 ^ 4) * 16);
+        if constexpr (kRowsInLane) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                a_voff[i] = (uint32_t)(((lane >> 3) + 8 * i) * s.a_ld * ES + (chunk0 ^ ((i & 1) << 2)) * 16);
+        } else {
+            a_voff[0] = (uint32_t)((lane >> 3) * s.a_ld * ES + chunk0 * 16);
+            a_voff[1] = (uint32_t)((lane >> 3) * s.a_ld * ES + (chunk0 ^ 4) * 16);
+        }
         if constexpr (B_KC) {
             b_base = b + (int64_t)(tile_n + wave * 32) * s.b_ld * ES;
             b_row_bytes = 8 * s.b_ld * ES;
             b_step_bytes = kRowBytes4;
-            b_voff[0] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
-            b_voff[1] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
+            if constexpr (kRowsInLane) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    b_voff[i] = (uint32_t)(((lane >> 3) + 8 * i) * s.b_ld * ES + (chunk0 ^ ((i & 1) << 2)) * 16);
+            } else {
+                b_voff[0] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
+                b_voff[1] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
+            }
         } else if constexpr (ES == 4) {
             // k-row of load i: k = 4 w + i, so (k/4)%4 = w % 4
             b_base = b + ((int64_t)(wave * 4) * s.b_ld + tile_n) * 4;
@@ -135,27 +162,30 @@ struct Loader4 {
             b_row_bytes = 2 * s.b_ld * 2;
             b_step_bytes = (int64_t)kBK4 * s.b_ld * 2;
 #pragma unroll
-            for (int v = 0; v < 2; ++v)
-                b_voff[v] = (uint32_t)(((lane >> 5) * s.b_ld + (chunk ^ (v << 3) ^ ((wave & 1) << 1)) * 8) * 2);
+            for (int v = 0; v < 4; ++v)
+                b_voff[v] = (uint32_t)((((lane >> 5) + 2 * v) * s.b_ld + (chunk ^ ((v & 1) << 3) ^ ((wave & 1) << 1)) * 8) * 2);
         }
     }
 
     // The wave's eight loads of one k-step (4 for A, 4 for B), then move the cursor on.
     __device__ __forceinline__ void issue(uint32_t stage_addr) {
-        const uint32_t sa = stage_addr + wave * 4096, sb = stage_addr + kATile4 + wave * 4096;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lds_dma16(a_base + i * a_row_bytes, a_voff[i & 1], sa + i * 1024);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], sb + i * 1024);
+        for (int q = 0; q < 8; ++q) issue_one(stage_addr + wave * 4096, q);
         advance();
     }
 
-    // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step; advance() after the eighth.
-    __device__ __forceinline__ void issue_one(uint32_t stage_addr, int q) {
-        if (q < 4) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], stage_addr + wave * 4096 + q * 1024);
-        else {
-            const int i = q - 4;
-            lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], stage_addr + kATile4 + wave * 4096 + i * 1024);
+    // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step into the stage whose LDS address plus
+    // this wave's 4 KiB is wave_stage; advance() after the eighth.
+    __device__ __forceinline__ void issue_one(uint32_t wave_stage, int q) {
+        if constexpr (kRowsInLane) {
+            if (q < 4) lds_dma16_k(a_base, a_voff[q], wave_stage, q * 1024);
+            else lds_dma16_k(b_base, b_voff[q - 4], wave_stage, kATile4 + (q - 4) * 1024);
+        } else {
+            if (q < 4) lds_dma16(a_base + q * a_row_bytes, a_voff[q & 1], wave_stage + q * 1024);
+            else {
+                const int i = q - 4;
+                lds_dma16(b_base + i * b_row_bytes, b_voff[i & 1], wave_stage + kATile4 + i * 1024);
+            }
         }
     }
     __device__ __forceinline__ void advance() {
@@ -171,10 +201,13 @@ struct Loader4 {
                     tile_m = tm * kBM4; tile_n = tn * kBN4;
                     total_seg = seg + 1;
                     point_at_segment();
-                } else seg = total_seg;
+                } else { point_at_segment(); seg = total_seg; }
             } else if (++seg < total_seg) point_at_segment();
+            else { --seg; point_at_segment(); ++seg; }
         }
     }
+    // (After the last step the cursor is back on the first k-step of the last tile: the 16-bit main loop
+    // issues its loads unconditionally, and those past the end must read addresses that exist.)
 
     __device__ __forceinline__ bool done() const { return seg >= total_seg; }
 };
@@ -288,6 +321,25 @@ struct Pipe4 {
     }
 
     __device__ __forceinline__ void run(Acc4& acc, int KT) {
+        if constexpr (es4<T>() == 2) run16(acc, KT); else run32(acc, KT);
+    }
+
+    // 16-bit operands.  A wave issues in order, and whatever stands between two matrix instructions holds
+    // the second one back unless it fits into the 16 cycles the first one occupies the pipe: so the row of
+    // four matrix instructions takes its other work in between them, at most three instructions at a time
+    // -- the A fragment of the next k-group after the first, the B fragment (first four rows) after the
+    // second, one of the wave's eight loads of step g+2 (second k-group only) after the third.  Cycle
+    // counters around the rows (timing builds): the rows after the barrier, with the loads, took 185 to 240
+    // cycles against 64 of matrix instructions while their scalar address arithmetic and a branch stood in
+    // front of the row; a k-step 2890 -> 2750 cycles with this order and the three-instruction loads.
+    // What a fragment read costs however it is placed is the return of its data, 1 KiB per read into the
+    // register file: about 8 cycles, in which the matrix pipe takes no operands -- 24 reads per wave and
+    // k-step, 19 % on top of the matrix instructions for this wave tile.
+    // The loads are issued unconditionally: past the last step they fetch the first k-step of the last
+    // tile again (Loader4::advance parks the cursor there) into a stage nobody reads, and run() does not
+    // return before they have landed.  More than one load per row costs more than it gains (the memory
+    // pipeline takes them slowly: all eight in the first four rows, k-step +3 %).
+    __device__ __forceinline__ void run16(Acc4& acc, int KT) {
         for (int kt = 0; kt < KT; ++kt, ++g) {
 #pragma unroll
             for (int kg = 0; kg < 2; ++kg) {
@@ -299,37 +351,33 @@ struct Pipe4 {
                     wait_vmcnt_imm<0>();
                     __syncthreads();
                 }
-                // The wave's eight loads of step g+2 go out one per row of matrix instructions
-                // (measured at 8192^3: one per row 0.865 ms, two 0.879, four or all at once 0.895).
-                const bool issuing = kg == 1 && !ld.done();
-                // Fragments of the next k-group come in between the rows of matrix instructions, one
-                // A and (first four rows) one B fragment per row: few enough in flight for the LDS
-                // counter (4 bits) to tell the old fragments from the new, and bursts of reads cost
-                // more (two pairs per row 0.878 ms, all up front 0.900).  In the last step the
-                // "next" fragments are stale data that nobody uses.
+                const uint32_t wave_stage = smem_addr + slot * kStageBytes4 + ld.wave * 4096;
+                // In the last step the "next" fragments are stale data that nobody uses.
                 const int nsl = kg == 0 ? slot : slot ^ 1, nkg = kg ^ 1;
+                const char* st = smem + nsl * kStageBytes4;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    if (issuing) {
-                        ld.issue_one(smem_addr + slot * kStageBytes4, i);
-                        if (i == 7) ld.advance();
+                    // boustrophedon: the B fragment carries over between rows
+                    auto mm = [&](int jj) { const int j = (i & 1) ? 3 - jj : jj; mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]); };
+                    mm(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    fa[nb][i] = read_frag16_kc(st, wm + i * 16, nkg);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mm(1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (i < 4) {
+                        if constexpr (B_KC) fb[nb][i] = read_frag16_kc(st + kATile4, wn + i * 16, nkg);
+                        else fb[nb][i] = read_frag16_mc(st + kATile4, wn + i * 16, nkg);
                     }
-                    read_pair(nb, nsl, nkg, i);
-                    if constexpr (es4<T>() == 4) {
-                        // four matrix instructions per accumulator and k-group: component-major, so
-                        // that instructions on one accumulator are four apart
-#pragma unroll
-                        for (int c = 0; c < 4; ++c)
-#pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
-                    } else {
-#pragma unroll
-                        for (int jj = 0; jj < 4; ++jj) {
-                            const int j = (i & 1) ? 3 - jj : jj;   // boustrophedon: the B fragment carries over between rows
-                            mfma16_step<T>(acc.t[i][j], fa[cb][i], fb[cb][j]);
-                        }
+                    __builtin_amdgcn_sched_barrier(0);
+                    mm(2);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (kg == 1) {
+                        ld.issue_one(wave_stage, i);
+                        if (i == 7 && !ld.done()) ld.advance();
                     }
+                    __builtin_amdgcn_sched_barrier(0);
+                    mm(3);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -337,6 +385,45 @@ struct Pipe4 {
         }
         // the matrix instructions are opaque to the compiler's hazard checks: let the last results
         // retire before the epilogue reads the accumulators
+        asm volatile("s_nop 15\n\ts_nop 15");
+        if (ld.done()) wait_vmcnt_imm<0>();   // the loads past the end: the epilogue may use the stages
+    }
+
+    // fp32 operands.
+    __device__ __forceinline__ void run32(Acc4& acc, int KT) {
+        for (int kt = 0; kt < KT; ++kt, ++g) {
+#pragma unroll
+            for (int kg = 0; kg < 2; ++kg) {
+                const int nb = kg ^ 1, cb = kg;
+                if (kg == 1) {
+                    wait_vmcnt_imm<0>();
+                    __syncthreads();
+                }
+                // The wave's eight loads of step g+2 go out one per row of matrix instructions.
+                const bool issuing = kg == 1 && !ld.done();
+                // Fragments of the next k-group come in between the rows of matrix instructions, one
+                // A and (first four rows) one B fragment per row: few enough in flight for the LDS
+                // counter (4 bits) to tell the old fragments from the new.
+                const int nsl = kg == 0 ? slot : slot ^ 1, nkg = kg ^ 1;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (issuing) {
+                        ld.issue_one(smem_addr + slot * kStageBytes4 + ld.wave * 4096, i);
+                        if (i == 7) ld.advance();
+                    }
+                    read_pair(nb, nsl, nkg, i);
+                    // four matrix instructions per accumulator and k-group: component-major, so
+                    // that instructions on one accumulator are four apart
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            mfma16_step_f32(acc.t[i][j], fa[cb][i][c], fb[cb][j][c]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            slot ^= 1;
+        }
         asm volatile("s_nop 15\n\ts_nop 15");
     }
 };

@@ -118,6 +118,9 @@ hipError_t launch_gemm4(const Gemm2Params& p, int batch, hipStream_t stream) {
     const int tiles = p.tiles_m * p.tiles_n;
     const int64_t total = (int64_t)tiles * nprod * batch;
     if (total <= 0 || total >= (1 << 30)) return hipErrorInvalidValue;
+    // the loader's lane offsets are 32-bit and reach over 32 rows of an operand
+    for (int s = 0; s < nprod; ++s)
+        if (p.seg[s].a_ld >= (int64_t(1) << 26) || p.seg[s].b_ld >= (int64_t(1) << 26)) return hipErrorInvalidValue;
     Gemm2Params q = p;
     // several small products at once: XCD-chunked numbering (see map_tile4)
     // (measured: grouped launch of config 4 1.585 -> 1.545 ms, two-level 8192^3 0.787 -> 0.766 ms)
