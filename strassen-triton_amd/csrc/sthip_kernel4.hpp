@@ -100,12 +100,19 @@ __device__ __forceinline__ void lds_dma16_k(const void* sbase, uint32_t voff, ui
     asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                  :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k) : "memory", "scc");
 }
+// The same under a lane mask that is all ones or zero: with no lane enabled the load is not executed
+// (no memory access, nothing to wait for).  The caller runs with all lanes enabled.
+__device__ __forceinline__ void lds_dma16_km(const void* sbase, uint32_t voff, uint32_t lds_addr, int k, uint32_t mask) {
+    asm volatile("s_mov_b32 exec_lo, %4\n\ts_mov_b32 exec_hi, %4\n\ts_add_u32 m0, %2, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
+                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k), "s"(mask) : "memory", "scc");
+}
 
 // 16-bit operands: the lane offset of load i includes the rows of load i (a_voff[i], b_voff[i]), so that
-// issuing a load in the main loop is three instructions (m0, a wait state, the load) and no scalar address
-// arithmetic: a wave issues in order, and a dozen scalar instructions and a branch per load held back the
-// matrix instructions behind them (measured: k-step 2890 -> 2750 cycles together with the row order of
-// Pipe4::run).  Lane offsets are 32-bit: 32 rows of the operand must span less than 4 GiB (the launcher
+// issuing a load in the main loop is m0, a wait state and the load (between two writes of the lane mask,
+// see Pipe4::run16) and no scalar address arithmetic: a wave issues in order, and a dozen scalar
+// instructions and a branch per load held back the matrix instructions behind them (measured: k-step
+// 2890 -> 2750 cycles together with the row order of Pipe4::run16).  Lane offsets are 32-bit: 32 rows of the operand must span less than 4 GiB (the launcher
 // checks).  fp32 operands keep one offset per load parity and add the rows to the base: that kernel has no
 // registers to spare.
 template <int ES, bool B_KC>
@@ -129,9 +136,9 @@ struct Loader4 {
         a_row_bytes = 8 * s.a_ld * ES;
         a_step_bytes = kRowBytes4;
         if constexpr (kRowsInLane) {
+            const uint32_t row = (uint32_t)(s.a_ld * ES), l8 = (uint32_t)(lane >> 3) * row;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                a_voff[i] = (uint32_t)(((lane >> 3) + 8 * i) * s.a_ld * ES + (chunk0 ^ ((i & 1) << 2)) * 16);
+            for (int i = 0; i < 4; ++i) a_voff[i] = l8 + 8 * i * row + (chunk0 ^ ((i & 1) << 2)) * 16;
         } else {
             a_voff[0] = (uint32_t)((lane >> 3) * s.a_ld * ES + chunk0 * 16);
             a_voff[1] = (uint32_t)((lane >> 3) * s.a_ld * ES + (chunk0 ^ 4) * 16);
@@ -141,9 +148,9 @@ struct Loader4 {
             b_row_bytes = 8 * s.b_ld * ES;
             b_step_bytes = kRowBytes4;
             if constexpr (kRowsInLane) {
+                const uint32_t row = (uint32_t)(s.b_ld * ES), l8 = (uint32_t)(lane >> 3) * row;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    b_voff[i] = (uint32_t)(((lane >> 3) + 8 * i) * s.b_ld * ES + (chunk0 ^ ((i & 1) << 2)) * 16);
+                for (int i = 0; i < 4; ++i) b_voff[i] = l8 + 8 * i * row + (chunk0 ^ ((i & 1) << 2)) * 16;
             } else {
                 b_voff[0] = (uint32_t)((lane >> 3) * s.b_ld * ES + chunk0 * 16);
                 b_voff[1] = (uint32_t)((lane >> 3) * s.b_ld * ES + (chunk0 ^ 4) * 16);
@@ -161,9 +168,9 @@ struct Loader4 {
             b_base = b + ((int64_t)(wave * 8) * s.b_ld + tile_n) * 2;
             b_row_bytes = 2 * s.b_ld * 2;
             b_step_bytes = (int64_t)kBK4 * s.b_ld * 2;
+            const uint32_t row = (uint32_t)(s.b_ld * 2), l32 = (uint32_t)(lane >> 5) * row;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                b_voff[v] = (uint32_t)((((lane >> 5) + 2 * v) * s.b_ld + (chunk ^ ((v & 1) << 3) ^ ((wave & 1) << 1)) * 8) * 2);
+            for (int v = 0; v < 4; ++v) b_voff[v] = l32 + 2 * v * row + (chunk ^ ((v & 1) << 3) ^ ((wave & 1) << 1)) * 16;
         }
     }
 
@@ -176,6 +183,11 @@ struct Loader4 {
 
     // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step into the stage whose LDS address plus
     // this wave's 4 KiB is wave_stage; advance() after the eighth.
+    // 16-bit main loop: the same under a lane mask (all ones, or zero once the loader has run dry).
+    __device__ __forceinline__ void issue_one_masked(uint32_t wave_stage, int q, uint32_t mask) {
+        if (q < 4) lds_dma16_km(a_base, a_voff[q], wave_stage, q * 1024, mask);
+        else lds_dma16_km(b_base, b_voff[q - 4], wave_stage, kATile4 + (q - 4) * 1024, mask);
+    }
     __device__ __forceinline__ void issue_one(uint32_t wave_stage, int q) {
         if constexpr (kRowsInLane) {
             if (q < 4) lds_dma16_k(a_base, a_voff[q], wave_stage, q * 1024);
@@ -201,13 +213,10 @@ struct Loader4 {
                     tile_m = tm * kBM4; tile_n = tn * kBN4;
                     total_seg = seg + 1;
                     point_at_segment();
-                } else { point_at_segment(); seg = total_seg; }
+                } else seg = total_seg;
             } else if (++seg < total_seg) point_at_segment();
-            else { --seg; point_at_segment(); ++seg; }
         }
     }
-    // (After the last step the cursor is back on the first k-step of the last tile: the 16-bit main loop
-    // issues its loads unconditionally, and those past the end must read addresses that exist.)
 
     __device__ __forceinline__ bool done() const { return seg >= total_seg; }
 };
@@ -335,10 +344,11 @@ struct Pipe4 {
     // What a fragment read costs however it is placed is the return of its data, 1 KiB per read into the
     // register file: about 8 cycles, in which the matrix pipe takes no operands -- 24 reads per wave and
     // k-step, 19 % on top of the matrix instructions for this wave tile.
-    // The loads are issued unconditionally: past the last step they fetch the first k-step of the last
-    // tile again (Loader4::advance parks the cursor there) into a stage nobody reads, and run() does not
-    // return before they have landed.  More than one load per row costs more than it gains (the memory
-    // pipeline takes them slowly: all eight in the first four rows, k-step +3 %).
+    // No load has a branch around it: once the loader has run dry (the last two steps of a workgroup's
+    // last tile) the loads are issued with no lane enabled, which executes nothing.  More than one load per
+    // row costs more than it gains (the memory pipeline takes them slowly: all eight in the first four rows,
+    // k-step +3 %); the loop written twice, with and without loads, makes the compiler spill around the
+    // tile's store (short tiles 10 % slower).
     __device__ __forceinline__ void run16(Acc4& acc, int KT) {
         for (int kt = 0; kt < KT; ++kt, ++g) {
 #pragma unroll
@@ -352,6 +362,7 @@ struct Pipe4 {
                     __syncthreads();
                 }
                 const uint32_t wave_stage = smem_addr + slot * kStageBytes4 + ld.wave * 4096;
+                const uint32_t live = (uint32_t)__builtin_amdgcn_readfirstlane(ld.done() ? 0 : -1);
                 // In the last step the "next" fragments are stale data that nobody uses.
                 const int nsl = kg == 0 ? slot : slot ^ 1, nkg = kg ^ 1;
                 const char* st = smem + nsl * kStageBytes4;
@@ -373,7 +384,7 @@ struct Pipe4 {
                     mm(2);
                     __builtin_amdgcn_sched_barrier(0);
                     if (kg == 1) {
-                        ld.issue_one(wave_stage, i);
+                        ld.issue_one_masked(wave_stage, i, live);
                         if (i == 7 && !ld.done()) ld.advance();
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -386,7 +397,6 @@ struct Pipe4 {
         // the matrix instructions are opaque to the compiler's hazard checks: let the last results
         // retire before the epilogue reads the accumulators
         asm volatile("s_nop 15\n\ts_nop 15");
-        if (ld.done()) wait_vmcnt_imm<0>();   // the loads past the end: the epilogue may use the stages
     }
 
     // fp32 operands.
