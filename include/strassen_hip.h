@@ -45,7 +45,8 @@ enum sthip_algo {
 
 /* General entry: C[b] (+)= A[b] x B[b] for b < batch, A is M x K, B is K x N, C is M x N.
  * stride*[3] = {batch, row, col} in elements; A and B need one unit stride among (row, col)
- * each (so NN / NT / TN / TT all work without copies).  in_dtype is the element type of A
+ * each (so NN / NT / TN / TT all work without copies; the other stride must stay below 2^26
+ * elements, or the call fails with STHIP_ERR_HIP).  in_dtype is the element type of A
  * and B; out_dtype is that of C and must equal in_dtype or be STHIP_F32.  Products
  * accumulate in fp32, operand sums are formed in fp32 and rounded once to in_dtype, the
  * recombination is done in fp32.  Sizes that are not multiples of 2^levels behave as if
