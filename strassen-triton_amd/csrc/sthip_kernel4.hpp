@@ -112,9 +112,9 @@ __device__ __forceinline__ void lds_dma16_km(const void* sbase, uint32_t voff, u
 // issuing a load in the main loop is m0, a wait state and the load (between two writes of the lane mask,
 // see Pipe4::run16) and no scalar address arithmetic: a wave issues in order, and a dozen scalar
 // instructions and a branch per load held back the matrix instructions behind them (measured: k-step
-// 2890 -> 2750 cycles together with the row order of Pipe4::run16).  Lane offsets are 32-bit: 32 rows of the operand must span less than 4 GiB (the launcher
-// checks).  fp32 operands keep one offset per load parity and add the rows to the base: that kernel has no
-// registers to spare.
+// 2890 -> 2750 cycles together with the row order of Pipe4::run16).  Lane offsets are 32-bit: 32 rows of
+// the operand must span less than 4 GiB (the launcher checks).  fp32 operands keep one offset per load
+// parity and add the rows to the base: that kernel has no registers to spare.
 template <int ES, bool B_KC>
 struct Loader4 {
     static constexpr bool kRowsInLane = ES == 2;
@@ -181,13 +181,13 @@ struct Loader4 {
         advance();
     }
 
-    // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step into the stage whose LDS address plus
-    // this wave's 4 KiB is wave_stage; advance() after the eighth.
-    // 16-bit main loop: the same under a lane mask (all ones, or zero once the loader has run dry).
+    // 16-bit main loop: load q under a lane mask (all ones, or zero once the loader has run dry).
     __device__ __forceinline__ void issue_one_masked(uint32_t wave_stage, int q, uint32_t mask) {
         if (q < 4) lds_dma16_km(a_base, a_voff[q], wave_stage, q * 1024, mask);
         else lds_dma16_km(b_base, b_voff[q - 4], wave_stage, kATile4 + (q - 4) * 1024, mask);
     }
+    // Load q (0..3 the A tile, 4..7 the B tile) of the next k-step into the stage whose LDS address plus
+    // this wave's 4 KiB is wave_stage; advance() after the eighth.
     __device__ __forceinline__ void issue_one(uint32_t wave_stage, int q) {
         if constexpr (kRowsInLane) {
             if (q < 4) lds_dma16_k(a_base, a_voff[q], wave_stage, q * 1024);
