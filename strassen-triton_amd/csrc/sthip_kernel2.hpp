@@ -21,6 +21,7 @@
 #include <stdint.h>
 
 #include "sthip_kernel.hpp"
+#include "sthip_prims.hpp"
 
 namespace sthip {
 
@@ -62,15 +63,6 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
 }
 
 typedef void __attribute__((address_space(3))) * lptr_t;
-
-// One 1 KiB direct-to-LDS load: lane L moves 16 bytes from sbase + voff to LDS byte address
-// lds_addr + 16 L.  Written as inline assembly on purpose: the compiler must not know that
-// LDS is being filled asynchronously, or it serialises every later LDS read behind
-// vmcnt(0); ordering is enforced by hand with wait_vmcnt() + the workgroup barrier.
-__device__ __forceinline__ void lds_dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
-}
 
 // Issues this wave's share (4 + 4 loads of 1 KiB) of one k-step into one LDS stage.
 // KC operand tile: 128 rows x 8 chunks of 16 bytes; the load that fills rows R..R+7 has lane

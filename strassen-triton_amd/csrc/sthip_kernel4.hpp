@@ -94,20 +94,6 @@ __device__ __forceinline__ void map_tile4(const Gemm2Params& P, int id, int& pro
 // n-contiguous fp32 B tile is 32 k-rows x 1024 bytes, one row per load: wave w loads k-rows
 // 4 w + i (i = 0..3), and slot s of row k holds chunk s ^ (((k / 4) % 4) * 4), so that the four k-rows a
 // fragment read touches (k = 4 g + c, lane group g) fall into different 64-byte bank groups.
-// lds_dma16 with the LDS address given as a uniform register plus a constant: one scalar instruction
-// for m0 and none for the global address (the rows of the load are part of the lane offset).
-__device__ __forceinline__ void lds_dma16_k(const void* sbase, uint32_t voff, uint32_t lds_addr, int k) {
-    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k) : "memory", "scc");
-}
-// The same under a lane mask that is all ones or zero: with no lane enabled the load is not executed
-// (no memory access, nothing to wait for).  The caller runs with all lanes enabled.
-__device__ __forceinline__ void lds_dma16_km(const void* sbase, uint32_t voff, uint32_t lds_addr, int k, uint32_t mask) {
-    asm volatile("s_mov_b32 exec_lo, %4\n\ts_mov_b32 exec_hi, %4\n\ts_add_u32 m0, %2, %3\n\ts_nop 0\n\t"
-                 "global_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k), "s"(mask) : "memory", "scc");
-}
-
 // 16-bit operands: the lane offset of load i includes the rows of load i (a_voff[i], b_voff[i]), so that
 // issuing a load in the main loop is m0, a wait state and the load (between two writes of the lane mask,
 // see Pipe4::run16) and no scalar address arithmetic: a wave issues in order, and a dozen scalar
@@ -246,9 +232,8 @@ __device__ __forceinline__ u32x4 read_frag16_mc(const char* tile, int sub, int k
     const int chunk = (sub >> 3) + ((l16 & 3) >> 1);
     const int slot = chunk ^ (((l16 >> 2) & 3) << 2) ^ ((grp & 1) << 1);
     const char* p = tile + k * 512 + slot * 16 + (l16 & 1) * 8;
-    typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * 512));
+    s16x4 lo = lds_read_tr16_b64(p);
+    s16x4 hi = lds_read_tr16_b64(p + 4 * 512);
     u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
     u32x4 r = {a[0], a[1], b[0], b[1]};
     return r;
@@ -265,22 +250,6 @@ __device__ __forceinline__ u32x4 read_frag16_mc_f32(const char* tile, int sub, i
 #pragma unroll
     for (int c = 0; c < 4; ++c) r[c] = *reinterpret_cast<const uint32_t*>(p + c * 1024);
     return r;
-}
-
-// acc (16 n x 16 m, transposed so that a lane holds four consecutive n) += B-fragment x A-fragment.
-// Written as assembly so that the accumulator is updated in place: given the builtin, the
-// register allocator puts result and addend in different registers and permutes the 64
-// accumulators back with ~180 register copies per k-step.
-// fp32: one v_mfma_f32_16x16x4 on component c of both fragments (k = 4 g + c for lane group g).
-__device__ __forceinline__ void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b) {
-    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
-}
-template <class T>
-__device__ __forceinline__ void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b) {
-    if constexpr (__is_same(T, bf16_t))
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
-    else
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
 }
 
 struct Acc4 {   // one 128 x 64 wave tile = 8 x 4 MFMA tiles = 128 registers
