@@ -485,6 +485,7 @@ __device__ __forceinline__ void store_tile4_lds(const Acc4& acc, const Gemm2Para
             *reinterpret_cast<u32x2*>(w + i * 2048 + waddr[j]) = o;
         }
     }
+    wave_exchange_point();
     // read back: lane -> row 8 r + lane / 8, 16-byte chunk lane % 8; the same wave wrote it, LDS keeps order
     const int r8 = lane >> 3, c16 = lane & 7;
     char* dst = Cb + ((int64_t)(row + r8) * P.c_rs + (col + 8 * c16)) * 2;
@@ -517,6 +518,7 @@ __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *reinterpret_cast<f32x4*>(w + (16 * ii + l16) * 256 + (((4 * j + q) ^ l16) * 16)) = acc.t[4 * h + ii][j];
+        wave_exchange_point();
         // read back: lane -> row 4 r + lane / 16 of the half, chunk lane % 16; same wave, LDS keeps order
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -524,6 +526,7 @@ __device__ __forceinline__ void store_tile4_lds_f32(const Acc4& acc, const Gemm2
             const f32x4 v = *reinterpret_cast<const f32x4*>(w + rl * 256 + ((l16 ^ (rl & 15)) * 16));
             store_hinted(v, reinterpret_cast<f32x4*>(dst + (int64_t)(64 * h + 4 * r) * P.c_rs), P.c_stream);
         }
+        wave_exchange_point();
     }
 }
 
@@ -557,12 +560,14 @@ __device__ __forceinline__ void store_tile4_own(const Acc4& acc, const Gemm2Para
                 *reinterpret_cast<u32x2*>(w + ii * 2048 + waddr[j]) = o;
             }
         }
+        wave_exchange_point();
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int rr = ((8 * r + r8) >> 1) & 7;
             const u32x4 v = *reinterpret_cast<const u32x4*>(w + (8 * r + r8) * 128 + ((c16 ^ rr) * 16));
             store_hinted(v, reinterpret_cast<u32x4*>(dst + (4 * h + r) * step), P.c_stream);
         }
+        wave_exchange_point();
     }
 }
 

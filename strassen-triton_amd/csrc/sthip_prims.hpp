@@ -37,6 +37,11 @@ __device__ __forceinline__ s16x4 lds_read_tr16_b64(const char* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
 }
 
+// The lanes of a wave execute in lockstep: what any lane has written to LDS before this point, every lane of
+// the same wave may read after it (the waits the compiler places order the accesses).  Nothing is generated
+// for it; the build of the kernels for the host synchronises the 64 threads of a wave here.
+__device__ __forceinline__ void wave_exchange_point() {}
+
 // acc (16 n x 16 m, transposed so that a lane holds four consecutive n) += B-fragment x A-fragment.
 // Written as assembly so that the accumulator is updated in place: given the builtin, the
 // register allocator puts result and addend in different registers and permutes the 64

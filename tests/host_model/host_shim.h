@@ -1,0 +1,39 @@
+// What the kernel headers under strassen-triton_amd/csrc need in order to compile for the host: the
+// HIP keywords as empty macros, the thread coordinates as thread-local variables, and the AMDGPU builtins
+// as functions.  One host thread plays one lane; kernel4_host.cpp holds the run-time side.
+#pragma once
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <algorithm>
+#include <vector>
+using std::min;
+using std::max;
+
+#define __device__
+#define __global__
+#define __host__
+#define __forceinline__ inline
+#define __launch_bounds__(x)
+#define __shared__
+
+struct HostDim3 { unsigned x, y, z; };
+extern thread_local HostDim3 threadIdx, blockIdx, gridDim, blockDim;
+
+void host_syncthreads();                 // barrier over the workgroup's threads
+void host_waitcnt(int imm);              // s_waitcnt: completes this lane's pending direct-to-LDS loads
+inline void __syncthreads() { host_syncthreads(); }
+inline void __builtin_amdgcn_s_waitcnt(int imm) { host_waitcnt(imm); }
+inline void __builtin_amdgcn_sched_barrier(int) {}
+inline void __builtin_amdgcn_sched_group_barrier(int, int, int) {}
+inline void __builtin_amdgcn_s_setprio(int) {}
+inline int __builtin_amdgcn_readfirstlane(int x) { return x; }   // only ever applied to uniform values
+
+// Builtins used by kernels that this build never instantiates: declared so that their code parses.
+typedef short host_s16x4 __attribute__((ext_vector_type(4)));
+template <class P> inline host_s16x4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(P) { abort(); }
+template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x2f32(A, B, V c, int, int, int) { abort(); }
+template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_f16(A, B, V c, int, int, int) { abort(); }
+template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, V c, int, int, int) { abort(); }

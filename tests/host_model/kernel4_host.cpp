@@ -1,0 +1,253 @@
+// The 256 x 256 kernels of sthip_kernel4.hpp run on the CPU, one host thread per lane.
+//
+// What is real: the kernels' own code -- tile numbering, loader cursors and lane offsets, LDS layouts and
+// swizzles, fragment reads, the order of loads, waits and barriers, the walking of tiles, the stores.
+// What is modelled here (in place of sthip_prims.hpp): a direct-to-LDS load copies 16 bytes per lane,
+// either at once or not before the lane's next s_waitcnt lets it (the two extremes of what the hardware
+// may do), after checking that source and destination lie inside the operand and the LDS allocation;
+// the matrix instructions and the transposing LDS read exchange their operands among the 64 threads of
+// a wave.  Inline assembly statements are stripped from the headers before this file is compiled (the
+// test does that); they only carry scheduling hints, waits that the builtins repeat, and the
+// instructions replaced here.
+#include <pthread.h>
+#include <deque>
+#include <thread>
+#include "host_shim.h"
+#include "sthip_kernel4.hpp"
+
+thread_local HostDim3 threadIdx, blockIdx, gridDim, blockDim;
+namespace sthip { alignas(1024) char smem[160 * 1024]; }
+
+namespace {
+constexpr int kLanes = 64, kWaves = 8, kThreadsWg = kLanes * kWaves;
+pthread_barrier_t g_wg_barrier, g_wave_barrier[kWaves];
+bool g_late = false;   // direct-to-LDS loads land at the last moment the waits allow
+struct Range { const char* p; size_t n; };
+std::vector<Range> g_global;   // what the kernel may read through the loader
+struct Pending { const char* src; char* dst; };
+thread_local std::deque<Pending> t_pending;
+thread_local int t_slot[3] = {0, 0, 0};
+sthip::u32x4 g_xa[kWaves][2][kLanes], g_xb[kWaves][2][kLanes];
+uint32_t g_fa[kWaves][2][kLanes], g_fb[kWaves][2][kLanes];
+const char* g_xp[kWaves][2][kLanes];
+
+[[noreturn]] void die(const char* what, const void* p) {
+    fprintf(stderr, "MODEL VIOLATION: %s (address %p, workgroup %u, thread %u)\n", what, p, blockIdx.x, threadIdx.x);
+    fflush(stderr);
+    _Exit(3);
+}
+void check_global(const char* p) {
+    for (const Range& r : g_global)
+        if (p >= r.p && p + 16 <= r.p + r.n) return;
+    die("direct-to-LDS load reads outside the operands", p);
+}
+void dma(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+    const int lane = threadIdx.x & 63;
+    const char* src = reinterpret_cast<const char*>(sbase) + voff;
+    char* dst = reinterpret_cast<char*>((uintptr_t)lds_addr) + 16 * lane;
+    check_global(src);
+    if (dst < sthip::smem || dst + 16 > sthip::smem + sizeof(sthip::smem)) die("direct-to-LDS load writes outside LDS", dst);
+    if (g_late) t_pending.push_back({src, dst});
+    else memcpy(dst, src, 16);
+}
+float as_float(uint32_t v, int idx, bool bf16) {
+    const uint16_t h = (uint16_t)(v >> (16 * idx));
+    if (bf16) return __builtin_bit_cast(float, (uint32_t)h << 16);
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+}  // namespace
+
+void host_syncthreads() { pthread_barrier_wait(&g_wg_barrier); }
+void host_waitcnt(int imm) {
+    const size_t n = (size_t)((imm & 0xF) | (((imm >> 14) & 3) << 4));   // vmcnt: this many loads may stay in flight
+    while (t_pending.size() > n) {
+        memcpy(t_pending.front().dst, t_pending.front().src, 16);
+        t_pending.pop_front();
+    }
+}
+
+namespace sthip {
+void lds_dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) { dma(sbase, voff, lds_addr); }
+void lds_dma16_k(const void* sbase, uint32_t voff, uint32_t lds_addr, int k) { dma(sbase, voff, lds_addr + (uint32_t)k); }
+void lds_dma16_km(const void* sbase, uint32_t voff, uint32_t lds_addr, int k, uint32_t mask) {
+    if (mask != 0 && mask != 0xffffffffu) die("lane mask of a load is neither all ones nor zero", sbase);
+    if (mask) dma(sbase, voff, lds_addr + (uint32_t)k);
+}
+void wave_exchange_point() { pthread_barrier_wait(&g_wave_barrier[threadIdx.x >> 6]); }
+// Lane i of a 16-lane group receives element i % 4 of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4.
+s16x4 lds_read_tr16_b64(const char* p) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot[0] ^= 1;
+    if (p < smem || p + 8 > smem + sizeof(smem)) die("transposing read outside LDS", p);
+    g_xp[wave][s][lane] = p;
+    pthread_barrier_wait(&g_wave_barrier[wave]);
+    const int base = lane & ~15, i = lane & 15;
+    s16x4 r;
+    for (int e = 0; e < 4; ++e) {
+        int16_t v;
+        memcpy(&v, g_xp[wave][s][base + 4 * e + i / 4] + 2 * (i % 4), 2);
+        r[e] = v;
+    }
+    return r;
+}
+// v_mfma_f32_16x16x32 as the kernel uses it: lane L accumulates, for m = L % 16 and n = 4 (L / 16) + e,
+// the sum over 32 k of A(m, k) B(n, k); the A fragment of row m holds k = 8 g .. 8 g + 7 in lane m + 16 g,
+// the B fragment of column n likewise.
+template <class T> void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot[1] ^= 1;
+    g_xa[wave][s][lane] = a;
+    g_xb[wave][s][lane] = b;
+    pthread_barrier_wait(&g_wave_barrier[wave]);
+    constexpr bool bf = __is_same(T, bf16_t);
+    const int m = lane & 15;
+    for (int e = 0; e < 4; ++e) {
+        const int n = 4 * (lane >> 4) + e;
+        float sum = 0.f;
+        for (int k = 0; k < 32; ++k) {
+            const u32x4& av = g_xa[wave][s][m + 16 * (k / 8)];
+            const u32x4& bv = g_xb[wave][s][n + 16 * (k / 8)];
+            sum += as_float(av[(k % 8) / 2], k % 2, bf) * as_float(bv[(k % 8) / 2], k % 2, bf);
+        }
+        acc[e] += sum;
+    }
+}
+template void mfma16_step<bf16_t>(f32x4&, const u32x4&, const u32x4&);
+template void mfma16_step<f16_t>(f32x4&, const u32x4&, const u32x4&);
+// v_mfma_f32_16x16x4_f32: k = lane group g; A(m, g) is the operand of lane m + 16 g.
+void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot[2] ^= 1;
+    g_fa[wave][s][lane] = a;
+    g_fb[wave][s][lane] = b;
+    pthread_barrier_wait(&g_wave_barrier[wave]);
+    const int m = lane & 15;
+    for (int e = 0; e < 4; ++e) {
+        const int n = 4 * (lane >> 4) + e;
+        float sum = 0.f;
+        for (int g = 0; g < 4; ++g)
+            sum += __builtin_bit_cast(float, g_fa[wave][s][m + 16 * g]) * __builtin_bit_cast(float, g_fb[wave][s][n + 16 * g]);
+        acc[e] += sum;
+    }
+}
+}  // namespace sthip
+
+namespace {
+using namespace sthip;
+
+template <class Kernel> void launch(Kernel kernel, const Gemm2Params& P, unsigned grid) {
+    for (unsigned wg = 0; wg < grid; ++wg) {
+        std::vector<std::thread> th;
+        th.reserve(kThreadsWg);
+        for (int t = 0; t < kThreadsWg; ++t)
+            th.emplace_back([=, &P] {
+                threadIdx = {(unsigned)t, 0, 0};
+                blockIdx = {wg, 0, 0};
+                gridDim = {grid, 1, 1};
+                blockDim = {(unsigned)kThreadsWg, 1, 1};
+                t_pending.clear();
+                kernel(P);
+                if (!t_pending.empty()) die("a lane ends with direct-to-LDS loads in flight", nullptr);
+            });
+        for (auto& x : th) x.join();
+    }
+}
+
+uint16_t to_half(float v, bool bf) {
+    if (bf) return (uint16_t)(__builtin_bit_cast(uint32_t, v) >> 16);
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+float from_half(uint16_t h, bool bf) { return as_float(h, 0, bf); }
+int small_int(uint32_t& state) {   // -1, 0, 1
+    state = state * 1664525u + 1013904223u;
+    return (int)((state >> 16) % 3) - 1;
+}
+
+// One configuration: `nprod` products C_p = A_p B_p of M x N x K each (M, N multiples of 256, K of the
+// k-step), on `grid` workgroups.  T: bf16_t, f16_t or float.  Returns the number of wrong elements.
+template <class T, bool B_KC>
+long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, bool walking, bool out_f32, bool accumulate) {
+    constexpr bool f32 = __is_same(T, float), bf = __is_same(T, bf16_t);
+    constexpr int ES = f32 ? 4 : 2;
+    const int es_out = (f32 || out_f32) ? 4 : 2;
+    const size_t a_elems = (size_t)M * K, b_elems = (size_t)K * N, c_elems = (size_t)M * N;
+    std::vector<char> A(nprod * a_elems * ES), B(nprod * b_elems * ES), C(nprod * c_elems * es_out);
+    std::vector<float> Af(nprod * a_elems), Bf(nprod * b_elems), C0(nprod * c_elems);
+    uint32_t seed = 12345u + (uint32_t)(M * 7 + N * 3 + K);
+    auto put = [&](std::vector<char>& buf, size_t i, float v) {
+        if (f32) memcpy(&buf[i * 4], &v, 4);
+        else { const uint16_t h = to_half(v, bf); memcpy(&buf[i * 2], &h, 2); }
+    };
+    for (size_t i = 0; i < Af.size(); ++i) { Af[i] = (float)small_int(seed); put(A, i, Af[i]); }
+    // B is stored k x n (n-contiguous) or n x k (k-contiguous); Bf is always indexed [p][k][n]
+    for (int p = 0; p < nprod; ++p)
+        for (int k = 0; k < K; ++k)
+            for (int n = 0; n < N; ++n) {
+                const float v = (float)small_int(seed);
+                Bf[p * b_elems + (size_t)k * N + n] = v;
+                put(B, p * b_elems + (B_KC ? (size_t)n * K + k : (size_t)k * N + n), v);
+            }
+    for (size_t i = 0; i < C0.size(); ++i) {
+        C0[i] = accumulate ? (float)small_int(seed) : 0.f;
+        if (es_out == 4) memcpy(&C[i * 4], &C0[i], 4);
+        else { const uint16_t h = to_half(accumulate ? C0[i] : 77.f, bf); memcpy(&C[i * 2], &h, 2); }
+    }
+    g_global = {{A.data(), A.size()}, {B.data(), B.size()}};
+
+    Gemm2Params P;
+    memset(&P, 0, sizeof(P));
+    for (int p = 0; p < nprod; ++p)
+        P.seg[p] = Seg2{A.data() + p * a_elems * ES, B.data() + p * b_elems * ES, K, B_KC ? K : N, 0, 0};
+    P.C = C.data(); P.c_rs = N; P.c_ps = (int64_t)c_elems; P.nprod = nprod;
+    P.Mh = M; P.Nh = N; P.Kh = K; P.tiles_m = M / 256; P.tiles_n = N / 256;
+    P.out_f32 = es_out == 4; P.accumulate = accumulate; P.group_m = 4; P.c_wide = 1; P.nbatch = 1;
+    P.xcd_chunks = 0;
+
+    long bad_total = 0;
+    for (int late = 0; late < 2; ++late) {
+        g_late = late != 0;
+        std::vector<char> Cw = C;
+        P.C = Cw.data();
+        memset(sthip::smem, 0xEE, sizeof(sthip::smem));
+        if (walking) launch(gemm4p_kernel<T, B_KC>, P, grid);
+        else launch(gemm4_kernel<T, B_KC>, P, (unsigned)(nprod * P.tiles_m * P.tiles_n));
+        long bad = 0;
+        for (int p = 0; p < nprod; ++p)
+            for (int m = 0; m < M; ++m)
+                for (int n = 0; n < N; ++n) {
+                    float want = C0[p * c_elems + (size_t)m * N + n];
+                    for (int k = 0; k < K; ++k) want += Af[p * a_elems + (size_t)m * K + k] * Bf[p * b_elems + (size_t)k * N + n];
+                    float got;
+                    const size_t i = p * c_elems + (size_t)m * N + n;
+                    if (es_out == 4) memcpy(&got, &Cw[i * 4], 4);
+                    else { uint16_t h; memcpy(&h, &Cw[i * 2], 2); got = from_half(h, bf); }
+                    if (got != want && bad++ < 5) fprintf(stderr, "  %s: C[%d][%d][%d] = %g, expected %g\n", name, p, m, n, got, want);
+                }
+        printf("%s  loads %s: %ld wrong of %zu\n", name, late ? "at the last moment" : "at once", bad, (size_t)nprod * c_elems);
+        fflush(stdout);
+        bad_total += bad;
+    }
+    return bad_total;
+}
+}  // namespace
+
+int main(int argc, char** argv) {
+    pthread_barrier_init(&g_wg_barrier, nullptr, kThreadsWg);
+    for (auto& b : g_wave_barrier) pthread_barrier_init(&b, nullptr, kLanes);
+    if ((uintptr_t)sthip::smem + sizeof(sthip::smem) > 0xffffffffull) { fprintf(stderr, "LDS stand-in above 4 GiB: link with -no-pie\n"); return 2; }
+    const int which = argc > 1 ? atoi(argv[1]) : -1;
+    long bad = 0;
+    int id = 0;
+    auto want = [&]() { return which < 0 || which == id++; };
+    // workgroups that walk their tiles: 4 tiles on 2 workgroups, odd number of k-steps
+    if (want()) bad += run_case<bf16_t, false>("walking bf16, B n-contiguous, 512x512x192, 2 workgroups", 1, 512, 512, 192, 2, true, false, false);
+    if (want()) bad += run_case<bf16_t, true>("walking bf16, B k-contiguous, 512x512x192, 2 workgroups", 1, 512, 512, 192, 2, true, false, false);
+    // two products side by side, 4 tiles on 3 workgroups (one walks two, tiles of different products)
+    if (want()) bad += run_case<f16_t, false>("walking fp16, two products of 256x512x128, 3 workgroups", 2, 256, 512, 128, 3, true, false, false);
+    // one tile per workgroup: plain, fp32 result, accumulating
+    if (want()) bad += run_case<bf16_t, true>("one tile per workgroup bf16, 256x512x64 (one k-step)", 1, 256, 512, 64, 0, false, false, false);
+    if (want()) bad += run_case<bf16_t, false>("one tile per workgroup bf16 -> fp32, 256x256x128", 1, 256, 256, 128, 0, false, true, false);
+    if (want()) bad += run_case<f16_t, true>("one tile per workgroup fp16, accumulating, 256x256x128", 1, 256, 256, 128, 0, false, false, true);
+    // fp32 operands (k-steps of 32)
+    if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
+    if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
+    printf("%s\n", bad ? "FAILED" : "ALL EXACT");
+    return bad ? 1 : 0;
+}

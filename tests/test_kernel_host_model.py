@@ -1,0 +1,118 @@
+"""The 256 x 256 kernels of strassen-triton_amd/csrc/sthip_kernel4.hpp compiled for the host and run on the
+CPU, one thread per lane (tests/host_model/kernel4_host.cpp).
+
+The kernel headers are the library's own; only their inline-assembly statements are taken out (scheduling
+hints, waits that builtins repeat, and the instructions of sthip_prims.hpp, which the host build replaces by
+functions that exchange operands among the threads of a wave and copy direct-to-LDS loads by hand, at once or
+at the last moment the waits allow, checking every source against the operands and every destination
+against the LDS allocation).  Products of small integers must come out exact for walking and one-tile-per-
+workgroup launches, both B layouts, bf16 / fp16 / fp32, plain, fp32-result and accumulating stores.  Two
+deliberately broken copies must be caught: one without the wait for the loads before the k-step's barrier,
+one that moves the loader's cursor before the last load of a step.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "strassen-triton_amd", "csrc")
+MODEL = os.path.join(ROOT, "tests", "host_model")
+HEADERS = ("sthip_kernel.hpp", "sthip_kernel2.hpp", "sthip_kernel3.hpp", "sthip_kernel4.hpp")
+
+
+def _clang():
+    for cand in (os.environ.get("STHIP_HOST_CXX"), "/opt/rocm/lib/llvm/bin/clang++", shutil.which("clang++")):
+        if cand and os.path.exists(cand):
+            return cand
+    return None
+
+
+def strip_asm(text: str) -> str:
+    """Replaces every `asm volatile(...);` statement by an empty statement."""
+    out, i = [], 0
+    pat = re.compile(r"\basm\s+volatile\s*\(")
+    while True:
+        m = pat.search(text, i)
+        if not m:
+            out.append(text[i:])
+            return "".join(out)
+        out.append(text[i:m.start()])
+        j, depth, in_str = m.end(), 1, False
+        while depth:
+            c = text[j]
+            if in_str:
+                if c == "\\":
+                    j += 1
+                elif c == '"':
+                    in_str = False
+            elif c == '"':
+                in_str = True
+            elif c == "(":
+                depth += 1
+            elif c == ")":
+                depth -= 1
+            j += 1
+        k = j
+        while text[k] in " \t":
+            k += 1
+        assert text[k] == ";", text[m.start():k + 20]
+        out.append("((void)0);")
+        i = k + 1
+
+
+def _build(tmp, name, mutate=None):
+    inc = os.path.join(tmp, name)
+    os.makedirs(inc)
+    for h in HEADERS:
+        text = strip_asm(open(os.path.join(CSRC, h)).read())
+        if mutate and h == "sthip_kernel4.hpp":
+            text = mutate(text)
+        open(os.path.join(inc, h), "w").write(text)
+    exe = os.path.join(inc, "kernel4_host")
+    cmd = [_clang(), "-std=c++17", "-O1", "-Wno-everything", "-no-pie", "-pthread", "-I", inc, "-I", MODEL,
+           "-I", os.path.join(ROOT, "include"), os.path.join(MODEL, "kernel4_host.cpp"), "-o", exe]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    return exe
+
+
+needs_clang = pytest.mark.skipif(_clang() is None, reason="no clang++ (the kernel headers use ext_vector_type)")
+
+
+def test_strip_asm_takes_out_whole_statements():
+    src = 'a(); asm volatile("s_nop 0\\n\\t(x)" :: "s"(f(1, 2)) : "memory");\nb = asm_volatile_count;'
+    assert strip_asm(src) == "a(); ((void)0);\nb = asm_volatile_count;"
+
+
+@needs_clang
+def test_kernels_exact_on_the_host(tmp_path):
+    exe = _build(str(tmp_path), "plain")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
+    assert len(lines) == 16 and all(": 0 wrong of" in l for l in lines), r.stdout
+    assert "ALL EXACT" in r.stdout
+
+
+def _drop_wait(text):
+    old = "                    wait_vmcnt_imm<0>();\n                    __syncthreads();\n                }\n                const uint32_t wave_stage"
+    assert old in text
+    return text.replace(old, "                    __syncthreads();\n                }\n                const uint32_t wave_stage", 1)
+
+
+def _advance_too_early(text):
+    old = "                        ld.issue_one_masked(wave_stage, i, live);\n                        if (i == 7 && !ld.done()) ld.advance();"
+    assert old in text
+    return text.replace(old, "                        if (i == 7 && !ld.done()) ld.advance();\n                        ld.issue_one_masked(wave_stage, i, live);", 1)
+
+
+@needs_clang
+@pytest.mark.parametrize("mutate", [_drop_wait, _advance_too_early], ids=["no wait before the barrier", "cursor moved before the last load"])
+def test_broken_copies_are_caught(tmp_path, mutate):
+    exe = _build(str(tmp_path), "broken", mutate)
+    r = subprocess.run([exe, "0"], capture_output=True, text=True, timeout=600)   # the first walking case is enough
+    assert r.returncode != 0, r.stdout
+    assert "MODEL VIOLATION" in r.stderr or "FAILED" in r.stdout
