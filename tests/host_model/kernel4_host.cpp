@@ -163,7 +163,7 @@ int small_int(uint32_t& state) {   // -1, 0, 1
 // One configuration: `nprod` products C_p = A_p B_p of M x N x K each (M, N multiples of 256, K of the
 // k-step), on `grid` workgroups.  T: bf16_t, f16_t or float.  Returns the number of wrong elements.
 template <class T, bool B_KC>
-long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, bool walking, bool out_f32, bool accumulate) {
+long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, bool walking, bool out_f32, bool accumulate, bool as_batch = false) {
     constexpr bool f32 = __is_same(T, float), bf = __is_same(T, bf16_t);
     constexpr int ES = f32 ? 4 : 2;
     const int es_out = (f32 || out_f32) ? 4 : 2;
@@ -196,8 +196,12 @@ long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, b
     for (int p = 0; p < nprod; ++p)
         P.seg[p] = Seg2{A.data() + p * a_elems * ES, B.data() + p * b_elems * ES, K, B_KC ? K : N, 0, 0};
     P.C = C.data(); P.c_rs = N; P.c_ps = (int64_t)c_elems; P.nprod = nprod;
+    if (as_batch) {   // the same operands addressed as batch entries of one product
+        P.seg[0].a_bs = (int64_t)a_elems; P.seg[0].b_bs = (int64_t)b_elems;
+        P.c_bs = (int64_t)c_elems; P.c_ps = 0; P.nprod = 1;
+    }
     P.Mh = M; P.Nh = N; P.Kh = K; P.tiles_m = M / 256; P.tiles_n = N / 256;
-    P.out_f32 = es_out == 4; P.accumulate = accumulate; P.group_m = 4; P.c_wide = 1; P.nbatch = 1;
+    P.out_f32 = es_out == 4; P.accumulate = accumulate; P.group_m = 4; P.c_wide = 1; P.nbatch = as_batch ? nprod : 1;
     P.xcd_chunks = 0;
 
     long bad_total = 0;
@@ -228,6 +232,25 @@ long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, b
 }
 }  // namespace
 
+// Every tile id of a launch must map to a different (batch, product, tile row, tile column), all of them in range.
+long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int xcd_chunks, int group_m) {
+    Gemm2Params P;
+    memset(&P, 0, sizeof(P));
+    P.tiles_m = tiles_m; P.tiles_n = tiles_n; P.nprod = nprod; P.nbatch = nbatch; P.xcd_chunks = xcd_chunks; P.group_m = group_m;
+    const int total = tiles_m * tiles_n * nprod * nbatch;
+    std::vector<char> seen((size_t)total, 0);
+    long bad = 0;
+    for (int id = 0; id < total; ++id) {
+        int prod, batch, tm, tn;
+        map_tile4(P, id, prod, batch, tm, tn);
+        if (prod < 0 || prod >= nprod || batch < 0 || batch >= nbatch || tm < 0 || tm >= tiles_m || tn < 0 || tn >= tiles_n) { ++bad; continue; }
+        const size_t key = (((size_t)batch * nprod + prod) * tiles_m + tm) * tiles_n + tn;
+        if (seen[key]++) ++bad;
+    }
+    printf("tile numbering %d x %d tiles, %d products, batch %d, chunks %d, group %d: %ld wrong of %d\n", tiles_m, tiles_n, nprod, nbatch, xcd_chunks, group_m, bad, total);
+    return bad;
+}
+
 int main(int argc, char** argv) {
     pthread_barrier_init(&g_wg_barrier, nullptr, kThreadsWg);
     for (auto& b : g_wave_barrier) pthread_barrier_init(&b, nullptr, kLanes);
@@ -241,6 +264,7 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case<bf16_t, true>("walking bf16, B k-contiguous, 512x512x192, 2 workgroups", 1, 512, 512, 192, 2, true, false, false);
     // two products side by side, 4 tiles on 3 workgroups (one walks two, tiles of different products)
     if (want()) bad += run_case<f16_t, false>("walking fp16, two products of 256x512x128, 3 workgroups", 2, 256, 512, 128, 3, true, false, false);
+    if (want()) bad += run_case<bf16_t, true>("walking bf16, batch of three 256x256x128, 2 workgroups", 3, 256, 256, 128, 2, true, false, false, true);
     // one tile per workgroup: plain, fp32 result, accumulating
     if (want()) bad += run_case<bf16_t, true>("one tile per workgroup bf16, 256x512x64 (one k-step)", 1, 256, 512, 64, 0, false, false, false);
     if (want()) bad += run_case<bf16_t, false>("one tile per workgroup bf16 -> fp32, 256x256x128", 1, 256, 256, 128, 0, false, true, false);
@@ -248,6 +272,18 @@ int main(int argc, char** argv) {
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
+    if (which < 0) {
+        // the launcher's choices: chunks for products of 32 / 64 / 128 tiles with tiles_m % 4 == 0 and >= 256 tiles in all
+        bad += check_tile_numbering(16, 16, 7, 1, 0, 4);
+        bad += check_tile_numbering(32, 32, 1, 1, 0, 8);
+        bad += check_tile_numbering(8, 8, 49, 1, 1, 4);
+        bad += check_tile_numbering(8, 16, 7, 1, 1, 4);
+        bad += check_tile_numbering(4, 8, 7, 8, 1, 4);
+        bad += check_tile_numbering(8, 4, 9, 1, 1, 4);     // 288 tiles: one chunk set of 256, the rest numbered plainly
+        bad += check_tile_numbering(3, 5, 7, 2, 0, 4);
+        bad += check_tile_numbering(32, 9, 1, 1, 0, 8);
+        bad += check_tile_numbering(5, 3, 1, 1, 0, 4);
+    }
     printf("%s\n", bad ? "FAILED" : "ALL EXACT");
     return bad ? 1 : 0;
 }

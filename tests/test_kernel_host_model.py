@@ -6,7 +6,8 @@ hints, waits that builtins repeat, and the instructions of sthip_prims.hpp, whic
 functions that exchange operands among the threads of a wave and copy direct-to-LDS loads by hand, at once or
 at the last moment the waits allow, checking every source against the operands and every destination
 against the LDS allocation).  Products of small integers must come out exact for walking and one-tile-per-
-workgroup launches, both B layouts, bf16 / fp16 / fp32, plain, fp32-result and accumulating stores.  Two
+workgroup launches, both B layouts, bf16 / fp16 / fp32, plain, fp32-result and accumulating stores, a batch;
+every tile id of a launch must map to a different tile (plain and XCD-chunked numbering).  Two
 deliberately broken copies must be caught: one without the wait for the loads before the k-step's barrier,
 one that moves the loader's cursor before the last load of a step.
 """
@@ -93,7 +94,7 @@ def test_kernels_exact_on_the_host(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
-    assert len(lines) == 16 and all(": 0 wrong of" in l for l in lines), r.stdout
+    assert len(lines) == 27 and all(": 0 wrong of" in l for l in lines), r.stdout   # 9 launches x 2 load timings, 9 tile numberings
     assert "ALL EXACT" in r.stdout
 
 
