@@ -46,13 +46,6 @@ struct Gemm6Params {
     int accumulate;        // C += product (plain products only)
 };
 
-// 16-byte global load whose completion the compiler does not track (see run6), and the dependency that
-// orders the uses of its result behind a hand-placed wait.
-__device__ __forceinline__ void gload16_6(f32x4& dst, const float* p) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
-}
-__device__ __forceinline__ void tie6(f32x4& x) { asm volatile("" : "+v"(x)); }
-
 __device__ __forceinline__ f32x4 combine6(f32x4 x, f32x4 y, int sign) {
     return sign > 0 ? x + y : x - y;
 }

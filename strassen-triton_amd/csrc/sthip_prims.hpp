@@ -1,4 +1,4 @@
-// The instructions the 256 x 256 kernel is built from that the compiler does not generate by itself:
+// The instructions the 256 x 256 and 64 x 64 kernels are built from that the compiler does not generate by itself:
 // direct-to-LDS loads, the transposing LDS read, the matrix instructions with their accumulator tied.
 // They are kept apart from the kernels so that a build for the host (tests/host_model/) can put
 // functions of its own in their place and run the kernels' index arithmetic on the CPU.
@@ -57,6 +57,14 @@ __device__ __forceinline__ void mfma16_step(f32x4& acc, const u32x4& a, const u3
     else
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
 }
+
+// 64 x 64 fp32 kernel (sthip_kernel6.hpp):
+// 16-byte global load whose completion the compiler does not track (see run6), and the dependency that
+// orders the uses of its result behind a hand-placed wait.
+__device__ __forceinline__ void gload16_6(f32x4& dst, const float* p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void tie6(f32x4& x) { asm volatile("" : "+v"(x)); }
 
 }  // namespace sthip
 

@@ -17,7 +17,7 @@ using std::max;
 #define __host__
 #define __forceinline__ inline
 #define __launch_bounds__(x)
-#define __shared__
+#define __shared__ static   // one copy for all threads: workgroups run one at a time (`extern __shared__` is rewritten to `extern`)
 
 struct HostDim3 { unsigned x, y, z; };
 extern thread_local HostDim3 threadIdx, blockIdx, gridDim, blockDim;
@@ -30,6 +30,13 @@ inline void __builtin_amdgcn_sched_barrier(int) {}
 inline void __builtin_amdgcn_sched_group_barrier(int, int, int) {}
 inline void __builtin_amdgcn_s_setprio(int) {}
 inline int __builtin_amdgcn_readfirstlane(int x) { return x; }   // only ever applied to uniform values
+
+void host_mfma_16x16x4(float a_inst, float b_inst, float* acc4);   // v_mfma_f32_16x16x4_f32 among the threads of a wave
+template <class V> inline V __builtin_amdgcn_mfma_f32_16x16x4f32(float a_inst, float b_inst, V acc, int, int, int) {
+    float r[4] = {acc[0], acc[1], acc[2], acc[3]};
+    host_mfma_16x16x4(a_inst, b_inst, r);
+    return V{r[0], r[1], r[2], r[3]};
+}
 
 // Builtins used by kernels that this build never instantiates: declared so that their code parses.
 typedef short host_s16x4 __attribute__((ext_vector_type(4)));

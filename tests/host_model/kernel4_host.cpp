@@ -14,6 +14,7 @@
 #include <thread>
 #include "host_shim.h"
 #include "sthip_kernel4.hpp"
+#include "sthip_kernel6.hpp"
 
 thread_local HostDim3 threadIdx, blockIdx, gridDim, blockDim;
 namespace sthip { alignas(1024) char smem[160 * 1024]; }
@@ -40,6 +41,11 @@ void check_global(const char* p) {
     for (const Range& r : g_global)
         if (p >= r.p && p + 16 <= r.p + r.n) return;
     die("direct-to-LDS load reads outside the operands", p);
+}
+void load16(const char* src, char* dst) {
+    check_global(src);
+    if (g_late) t_pending.push_back({src, dst});
+    else memcpy(dst, src, 16);
 }
 void dma(const void* sbase, uint32_t voff, uint32_t lds_addr) {
     const int lane = threadIdx.x & 63;
@@ -112,6 +118,7 @@ template <class T> void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b) 
 }
 template void mfma16_step<bf16_t>(f32x4&, const u32x4&, const u32x4&);
 template void mfma16_step<f16_t>(f32x4&, const u32x4&, const u32x4&);
+void gload16_6(f32x4& dst, const float* p) { load16(reinterpret_cast<const char*>(p), reinterpret_cast<char*>(&dst)); }
 // v_mfma_f32_16x16x4_f32: k = lane group g; A(m, g) is the operand of lane m + 16 g.
 void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot[2] ^= 1;
@@ -129,19 +136,29 @@ void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b) {
 }
 }  // namespace sthip
 
+// The builtin form (64 x 64 kernel): the instruction's first operand indexes the result's rows, which the
+// kernel uses for n, its second the columns (m): the same exchange as mfma16_step_f32 with a = second, b = first.
+void host_mfma_16x16x4(float a_inst, float b_inst, float* acc4) {
+    sthip::f32x4 acc = {acc4[0], acc4[1], acc4[2], acc4[3]};
+    sthip::mfma16_step_f32(acc, __builtin_bit_cast(uint32_t, b_inst), __builtin_bit_cast(uint32_t, a_inst));
+    for (int e = 0; e < 4; ++e) acc4[e] = acc[e];
+}
+
 namespace {
 using namespace sthip;
 
-template <class Kernel> void launch(Kernel kernel, const Gemm2Params& P, unsigned grid) {
+template <class Kernel, class Params> void launch(Kernel kernel, const Params& P, unsigned grid, int threads = kThreadsWg) {
+    pthread_barrier_destroy(&g_wg_barrier);
+    pthread_barrier_init(&g_wg_barrier, nullptr, threads);
     for (unsigned wg = 0; wg < grid; ++wg) {
         std::vector<std::thread> th;
-        th.reserve(kThreadsWg);
-        for (int t = 0; t < kThreadsWg; ++t)
+        th.reserve(threads);
+        for (int t = 0; t < threads; ++t)
             th.emplace_back([=, &P] {
                 threadIdx = {(unsigned)t, 0, 0};
                 blockIdx = {wg, 0, 0};
                 gridDim = {grid, 1, 1};
-                blockDim = {(unsigned)kThreadsWg, 1, 1};
+                blockDim = {(unsigned)threads, 1, 1};
                 t_pending.clear();
                 kernel(P);
                 if (!t_pending.empty()) die("a lane ends with direct-to-LDS loads in flight", nullptr);
@@ -232,6 +249,58 @@ long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, b
 }
 }  // namespace
 
+// 64 x 64 fp32 kernel: `nprod` products C_q = (A0 +- A1)(B0 +- B1) (or single blocks) of M x N x K.
+template <bool B_KC>
+long run_case6(const char* name, int nprod, int M, int N, int K, bool sums, bool accumulate) {
+    const size_t a_elems = (size_t)M * K, b_elems = (size_t)K * N, c_elems = (size_t)M * N;
+    std::vector<float> A(2 * nprod * a_elems), Bs(2 * nprod * b_elems), Bf(2 * nprod * b_elems), C0(nprod * c_elems);
+    uint32_t seed = 999u + (uint32_t)(M + 3 * N + 7 * K);
+    for (auto& v : A) v = (float)small_int(seed);
+    for (int p = 0; p < 2 * nprod; ++p)
+        for (int k = 0; k < K; ++k)
+            for (int n = 0; n < N; ++n) {
+                const float v = (float)small_int(seed);
+                Bf[p * b_elems + (size_t)k * N + n] = v;
+                Bs[p * b_elems + (B_KC ? (size_t)n * K + k : (size_t)k * N + n)] = v;
+            }
+    for (auto& v : C0) v = accumulate ? (float)small_int(seed) : 55.f;
+    g_global = {{reinterpret_cast<const char*>(A.data()), A.size() * 4}, {reinterpret_cast<const char*>(Bs.data()), Bs.size() * 4}};
+    Gemm6Params P;
+    memset(&P, 0, sizeof(P));
+    std::vector<int> sa(nprod), sb(nprod);
+    for (int q = 0; q < nprod; ++q) {
+        sa[q] = sums ? (q % 3 == 0 ? 1 : q % 3 == 1 ? -1 : 0) : 0;
+        sb[q] = sums ? (q % 4 == 0 ? -1 : q % 4 == 1 ? 0 : 1) : 0;
+        P.a[q] = Op6{A.data() + (2 * q) * a_elems, A.data() + (2 * q + 1) * a_elems, K, sa[q], 0};
+        P.b[q] = Op6{Bs.data() + (2 * q) * b_elems, Bs.data() + (2 * q + 1) * b_elems, B_KC ? K : N, sb[q], 0};
+    }
+    P.c_rs = N; P.c_ps = (int64_t)c_elems; P.Kh = K; P.tiles_m = M / 64; P.tiles_n = N / 64; P.nprod = nprod; P.accumulate = accumulate;
+    long bad_total = 0;
+    for (int late = 0; late < 2; ++late) {
+        g_late = late != 0;
+        std::vector<float> Cw = C0;
+        P.C = Cw.data();
+        launch(gemm6_kernel<B_KC>, P, (unsigned)(nprod * P.tiles_m * P.tiles_n), 256);
+        long bad = 0;
+        for (int q = 0; q < nprod; ++q)
+            for (int m = 0; m < M; ++m)
+                for (int n = 0; n < N; ++n) {
+                    float want = accumulate ? C0[q * c_elems + (size_t)m * N + n] : 0.f;
+                    for (int k = 0; k < K; ++k) {
+                        const float a = A[(2 * q) * a_elems + (size_t)m * K + k] + sa[q] * A[(2 * q + 1) * a_elems + (size_t)m * K + k];
+                        const float b = Bf[(2 * q) * b_elems + (size_t)k * N + n] + sb[q] * Bf[(2 * q + 1) * b_elems + (size_t)k * N + n];
+                        want += a * b;
+                    }
+                    const float got = Cw[q * c_elems + (size_t)m * N + n];
+                    if (got != want && bad++ < 5) fprintf(stderr, "  %s: C[%d][%d][%d] = %g, expected %g\n", name, q, m, n, got, want);
+                }
+        printf("%s  loads %s: %ld wrong of %zu\n", name, late ? "at the last moment" : "at once", bad, (size_t)nprod * c_elems);
+        fflush(stdout);
+        bad_total += bad;
+    }
+    return bad_total;
+}
+
 // Every tile id of a launch must map to a different (batch, product, tile row, tile column), all of them in range.
 long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int xcd_chunks, int group_m) {
     Gemm2Params P;
@@ -269,6 +338,11 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case<bf16_t, true>("one tile per workgroup bf16, 256x512x64 (one k-step)", 1, 256, 512, 64, 0, false, false, false);
     if (want()) bad += run_case<bf16_t, false>("one tile per workgroup bf16 -> fp32, 256x256x128", 1, 256, 256, 128, 0, false, true, false);
     if (want()) bad += run_case<f16_t, true>("one tile per workgroup fp16, accumulating, 256x256x128", 1, 256, 256, 128, 0, false, false, true);
+    // the 64 x 64 fp32 kernel: one product, and seven with operand sums formed in the loads
+    if (want()) bad += run_case6<false>("64x64 fp32, one product 128x192x128, B n-contiguous", 1, 128, 192, 128, false, false);
+    if (want()) bad += run_case6<true>("64x64 fp32, one product 128x128x64, B k-contiguous, accumulating", 1, 128, 128, 64, false, true);
+    if (want()) bad += run_case6<false>("64x64 fp32, seven products 128x128x128 of operand sums, B n-contiguous", 7, 128, 128, 128, true, false);
+    if (want()) bad += run_case6<true>("64x64 fp32, seven products 64x128x64 of operand sums, B k-contiguous", 7, 64, 128, 64, true, false);
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);

@@ -9,4 +9,6 @@ s16x4 lds_read_tr16_b64(const char* p);
 void mfma16_step_f32(f32x4& acc, uint32_t a, uint32_t b);
 template <class T> void mfma16_step(f32x4& acc, const u32x4& a, const u32x4& b);
 void wave_exchange_point();
+void gload16_6(f32x4& dst, const float* p);
+inline void tie6(f32x4&) {}
 }  // namespace sthip

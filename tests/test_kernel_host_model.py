@@ -1,5 +1,5 @@
-"""The 256 x 256 kernels of strassen-triton_amd/csrc/sthip_kernel4.hpp compiled for the host and run on the
-CPU, one thread per lane (tests/host_model/kernel4_host.cpp).
+"""The 256 x 256 kernels of strassen-triton_amd/csrc/sthip_kernel4.hpp and the 64 x 64 fp32 kernel of
+sthip_kernel6.hpp compiled for the host and run on the CPU, one thread per lane (tests/host_model/kernel4_host.cpp).
 
 The kernel headers are the library's own; only their inline-assembly statements are taken out (scheduling
 hints, waits that builtins repeat, and the instructions of sthip_prims.hpp, which the host build replaces by
@@ -8,8 +8,9 @@ at the last moment the waits allow, checking every source against the operands a
 against the LDS allocation).  Products of small integers must come out exact for walking and one-tile-per-
 workgroup launches, both B layouts, bf16 / fp16 / fp32, plain, fp32-result and accumulating stores, a batch;
 every tile id of a launch must map to a different tile (plain and XCD-chunked numbering).  Two
-deliberately broken copies must be caught: one without the wait for the loads before the k-step's barrier,
-one that moves the loader's cursor before the last load of a step.
+deliberately broken copies of the large kernel must be caught: one without the wait for the loads before the
+k-step's barrier, one that moves the loader's cursor before the last load of a step; and one of the small
+kernel that waits one load short.
 """
 import os
 import re
@@ -21,7 +22,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "strassen-triton_amd", "csrc")
 MODEL = os.path.join(ROOT, "tests", "host_model")
-HEADERS = ("sthip_kernel.hpp", "sthip_kernel2.hpp", "sthip_kernel3.hpp", "sthip_kernel4.hpp")
+HEADERS = ("sthip_kernel.hpp", "sthip_kernel2.hpp", "sthip_kernel3.hpp", "sthip_kernel4.hpp", "sthip_kernel6.hpp")
 
 
 def _clang():
@@ -64,12 +65,12 @@ def strip_asm(text: str) -> str:
         i = k + 1
 
 
-def _build(tmp, name, mutate=None):
+def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp"):
     inc = os.path.join(tmp, name)
     os.makedirs(inc)
     for h in HEADERS:
-        text = strip_asm(open(os.path.join(CSRC, h)).read())
-        if mutate and h == "sthip_kernel4.hpp":
+        text = strip_asm(open(os.path.join(CSRC, h)).read()).replace("extern __shared__", "extern")
+        if mutate and h == mutate_header:
             text = mutate(text)
         open(os.path.join(inc, h), "w").write(text)
     exe = os.path.join(inc, "kernel4_host")
@@ -94,7 +95,7 @@ def test_kernels_exact_on_the_host(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
-    assert len(lines) == 27 and all(": 0 wrong of" in l for l in lines), r.stdout   # 9 launches x 2 load timings, 9 tile numberings
+    assert len(lines) == 35 and all(": 0 wrong of" in l for l in lines), r.stdout   # 13 launches x 2 load timings, 9 tile numberings
     assert "ALL EXACT" in r.stdout
 
 
@@ -110,10 +111,18 @@ def _advance_too_early(text):
     return text.replace(old, "                        if (i == 7 && !ld.done()) ld.advance();\n                        ld.issue_one_masked(wave_stage, i, live);", 1)
 
 
+def _short_wait6(text):   # 64 x 64 kernel: one load of the older register set may still be in flight when it is used
+    old = "        wait_vmcnt_imm<kLoadsPerSet>();\n"
+    assert old in text
+    return text.replace(old, "        wait_vmcnt_imm<kLoadsPerSet + 1>();\n", 1)
+
+
 @needs_clang
-@pytest.mark.parametrize("mutate", [_drop_wait, _advance_too_early], ids=["no wait before the barrier", "cursor moved before the last load"])
-def test_broken_copies_are_caught(tmp_path, mutate):
-    exe = _build(str(tmp_path), "broken", mutate)
-    r = subprocess.run([exe, "0"], capture_output=True, text=True, timeout=600)   # the first walking case is enough
+@pytest.mark.parametrize("mutate, header, case", [(_drop_wait, "sthip_kernel4.hpp", "0"), (_advance_too_early, "sthip_kernel4.hpp", "0"),
+                                                  (_short_wait6, "sthip_kernel6.hpp", "9")],
+                         ids=["no wait before the barrier", "cursor moved before the last load", "64x64: wait one load short"])
+def test_broken_copies_are_caught(tmp_path, mutate, header, case):
+    exe = _build(str(tmp_path), "broken", mutate, header)
+    r = subprocess.run([exe, case], capture_output=True, text=True, timeout=600)   # one launch is enough
     assert r.returncode != 0, r.stdout
     assert "MODEL VIOLATION" in r.stderr or "FAILED" in r.stdout
