@@ -180,7 +180,7 @@ int small_int(uint32_t& state) {   // -1, 0, 1
 // One configuration: `nprod` products C_p = A_p B_p of M x N x K each (M, N multiples of 256, K of the
 // k-step), on `grid` workgroups.  T: bf16_t, f16_t or float.  Returns the number of wrong elements.
 template <class T, bool B_KC>
-long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, bool walking, bool out_f32, bool accumulate, bool as_batch = false) {
+long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, bool walking, bool out_f32, bool accumulate, bool as_batch = false, bool c_wide = true) {
     constexpr bool f32 = __is_same(T, float), bf = __is_same(T, bf16_t);
     constexpr int ES = f32 ? 4 : 2;
     const int es_out = (f32 || out_f32) ? 4 : 2;
@@ -218,7 +218,7 @@ long run_case(const char* name, int nprod, int M, int N, int K, unsigned grid, b
         P.c_bs = (int64_t)c_elems; P.c_ps = 0; P.nprod = 1;
     }
     P.Mh = M; P.Nh = N; P.Kh = K; P.tiles_m = M / 256; P.tiles_n = N / 256;
-    P.out_f32 = es_out == 4; P.accumulate = accumulate; P.group_m = 4; P.c_wide = 1; P.nbatch = as_batch ? nprod : 1;
+    P.out_f32 = es_out == 4; P.accumulate = accumulate; P.group_m = 4; P.c_wide = c_wide ? 1 : 0; P.nbatch = as_batch ? nprod : 1;
     P.xcd_chunks = 0;
 
     long bad_total = 0;
@@ -338,6 +338,9 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case<bf16_t, true>("one tile per workgroup bf16, 256x512x64 (one k-step)", 1, 256, 512, 64, 0, false, false, false);
     if (want()) bad += run_case<bf16_t, false>("one tile per workgroup bf16 -> fp32, 256x256x128", 1, 256, 256, 128, 0, false, true, false);
     if (want()) bad += run_case<f16_t, true>("one tile per workgroup fp16, accumulating, 256x256x128", 1, 256, 256, 128, 0, false, false, true);
+    if (want()) bad += run_case<bf16_t, false>("one tile per workgroup bf16, store straight from the accumulators, 256x256x64", 1, 256, 256, 64, 0, false, false, false, false, false);
+    if (want()) bad += run_case<bf16_t, true>("one tile per workgroup bf16 -> fp32, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
+    if (want()) bad += run_case<f16_t, true>("walking fp16, three tiles of two k-steps on 2 workgroups, 768x256x128", 1, 768, 256, 128, 2, true, false, false);
     // the 64 x 64 fp32 kernel: one product, and seven with operand sums formed in the loads
     if (want()) bad += run_case6<false>("64x64 fp32, one product 128x192x128, B n-contiguous", 1, 128, 192, 128, false, false);
     if (want()) bad += run_case6<true>("64x64 fp32, one product 128x128x64, B k-contiguous, accumulating", 1, 128, 128, 64, false, true);

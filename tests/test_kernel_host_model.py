@@ -95,7 +95,7 @@ def test_kernels_exact_on_the_host(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
-    assert len(lines) == 35 and all(": 0 wrong of" in l for l in lines), r.stdout   # 13 launches x 2 load timings, 9 tile numberings
+    assert len(lines) == 41 and all(": 0 wrong of" in l for l in lines), r.stdout   # 16 launches x 2 load timings, 9 tile numberings
     assert "ALL EXACT" in r.stdout
 
 
@@ -119,7 +119,7 @@ def _short_wait6(text):   # 64 x 64 kernel: one load of the older register set m
 
 @needs_clang
 @pytest.mark.parametrize("mutate, header, case", [(_drop_wait, "sthip_kernel4.hpp", "0"), (_advance_too_early, "sthip_kernel4.hpp", "0"),
-                                                  (_short_wait6, "sthip_kernel6.hpp", "9")],
+                                                  (_short_wait6, "sthip_kernel6.hpp", "12")],
                          ids=["no wait before the barrier", "cursor moved before the last load", "64x64: wait one load short"])
 def test_broken_copies_are_caught(tmp_path, mutate, header, case):
     exe = _build(str(tmp_path), "broken", mutate, header)
