@@ -65,7 +65,7 @@ def strip_asm(text: str) -> str:
         i = k + 1
 
 
-def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp"):
+def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp", extra=()):
     inc = os.path.join(tmp, name)
     os.makedirs(inc)
     for h in HEADERS:
@@ -74,7 +74,7 @@ def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp"):
             text = mutate(text)
         open(os.path.join(inc, h), "w").write(text)
     exe = os.path.join(inc, "kernel4_host")
-    cmd = [_clang(), "-std=c++17", "-O1", "-Wno-everything", "-no-pie", "-pthread", "-I", inc, "-I", MODEL,
+    cmd = [_clang(), "-std=c++17", "-O1", "-Wno-everything", "-no-pie", "-pthread", *extra, "-I", inc, "-I", MODEL,
            "-I", os.path.join(ROOT, "include"), os.path.join(MODEL, "kernel4_host.cpp"), "-o", exe]
     r = subprocess.run(cmd, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
@@ -97,6 +97,36 @@ def test_kernels_exact_on_the_host(tmp_path):
     lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
     assert len(lines) == 41 and all(": 0 wrong of" in l for l in lines), r.stdout   # 16 launches x 2 load timings, 9 tile numberings
     assert "ALL EXACT" in r.stdout
+
+
+@needs_clang
+def test_no_data_race_under_thread_sanitizer(tmp_path):
+    """Lanes are threads, barriers are barriers, a direct-to-LDS load is a write by the issuing thread: an LDS
+    buffer that is overwritten while another wave may still read it, or read before its barrier, is a data
+    race that ThreadSanitizer reports whatever the timing of this run was."""
+    try:
+        exe = _build(str(tmp_path), "tsan", extra=("-g", "-fsanitize=thread"))
+    except AssertionError as e:   # no ThreadSanitizer runtime with this compiler
+        pytest.skip(str(e)[-300:])
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
+    assert "ThreadSanitizer" not in r.stderr, r.stderr[:4000]
+    assert r.returncode == 0 and "ALL EXACT" in r.stdout, r.stdout[-2000:]
+
+
+def _drop_barrier(text):
+    old = "                    wait_vmcnt_imm<0>();\n                    __syncthreads();\n                }\n                const uint32_t wave_stage"
+    assert old in text
+    return text.replace(old, "                    wait_vmcnt_imm<0>();\n                }\n                const uint32_t wave_stage", 1)
+
+
+@needs_clang
+def test_thread_sanitizer_sees_a_missing_barrier(tmp_path):
+    try:
+        exe = _build(str(tmp_path), "tsan_broken", _drop_barrier, extra=("-g", "-fsanitize=thread"))
+    except AssertionError as e:
+        pytest.skip(str(e)[-300:])
+    r = subprocess.run([exe, "0"], capture_output=True, text=True, timeout=900)
+    assert "ThreadSanitizer: data race" in r.stderr
 
 
 def _drop_wait(text):
