@@ -142,9 +142,8 @@ __device__ __forceinline__ u32x4 read_frag2(const char* tile, int sub, int kg) {
         const int chunk = (sub >> 3) + (grp & 1) * 2 + ((l16 & 3) >> 1);
         const int slot = chunk ^ (((l16 >> 2) & 3) << 2);
         const char* p = tile + k * 256 + slot * 16 + (l16 & 1) * 8;
-        typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * 256));
+        s16x4 lo = lds_read_tr16_b64(p);
+        s16x4 hi = lds_read_tr16_b64(p + 4 * 256);
         u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
         u32x4 r = {a[0], a[1], b[0], b[1]};
         return r;

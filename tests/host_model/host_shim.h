@@ -38,9 +38,31 @@ template <class V> inline V __builtin_amdgcn_mfma_f32_16x16x4f32(float a_inst, f
     return V{r[0], r[1], r[2], r[3]};
 }
 
-// Builtins used by kernels that this build never instantiates: declared so that their code parses.
+// v_mfma_f32_32x32x16 (16-bit operands, eight per lane) and v_mfma_f32_32x32x2 (fp32, one per lane) among the
+// threads of a wave; `halves` are the raw 16-bit patterns.
+void host_mfma_32x32x16(const uint16_t a_inst[8], const uint16_t b_inst[8], float acc16[16], bool bf16);
+void host_mfma_32x32x2(float a_inst, float b_inst, float acc16[16]);
+template <class A, class V> inline V host_mfma16_wrap(A a, A b, V acc, bool bf16) {
+    uint16_t ha[8], hb[8];
+    float r[16];
+    memcpy(ha, &a, 16); memcpy(hb, &b, 16);
+    for (int e = 0; e < 16; ++e) r[e] = acc[e];
+    host_mfma_32x32x16(ha, hb, r, bf16);
+    V o;
+    for (int e = 0; e < 16; ++e) o[e] = r[e];
+    return o;
+}
+template <class A, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_bf16(A a, A b, V acc, int, int, int) { return host_mfma16_wrap(a, b, acc, true); }
+template <class A, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_f16(A a, A b, V acc, int, int, int) { return host_mfma16_wrap(a, b, acc, false); }
+template <class V> inline V __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float b, V acc, int, int, int) {
+    float r[16];
+    for (int e = 0; e < 16; ++e) r[e] = acc[e];
+    host_mfma_32x32x2(a, b, r);
+    V o;
+    for (int e = 0; e < 16; ++e) o[e] = r[e];
+    return o;
+}
+
+// Used directly by the fused 128 x 128 kernel of sthip_kernel.hpp, which this build does not run.
 typedef short host_s16x4 __attribute__((ext_vector_type(4)));
 template <class P> inline host_s16x4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(P) { abort(); }
-template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x2f32(A, B, V c, int, int, int) { abort(); }
-template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_f16(A, B, V c, int, int, int) { abort(); }
-template <class A, class B, class V> inline V __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, V c, int, int, int) { abort(); }

@@ -144,6 +144,38 @@ void host_mfma_16x16x4(float a_inst, float b_inst, float* acc4) {
     for (int e = 0; e < 4; ++e) acc4[e] = acc[e];
 }
 
+// v_mfma_f32_32x32x16: the first operand's lane L holds row L % 32 of a 32 x 16 block, k = 8 (L / 32) .. + 7,
+// the second's column L % 32 likewise; lane L receives, in element e, row 8 (e / 4) + 4 (L / 32) + e % 4 of
+// column L % 32.
+uint16_t g_ha[kWaves][2][kLanes][8], g_hb[kWaves][2][kLanes][8];
+float g_sa[kWaves][2][kLanes], g_sb[kWaves][2][kLanes];
+thread_local int t_slot32[2] = {0, 0};
+void host_mfma_32x32x16(const uint16_t a_inst[8], const uint16_t b_inst[8], float acc16[16], bool bf16) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot32[0] ^= 1;
+    memcpy(g_ha[wave][s][lane], a_inst, 16);
+    memcpy(g_hb[wave][s][lane], b_inst, 16);
+    pthread_barrier_wait(&g_wave_barrier[wave]);
+    const int col = lane & 31;
+    for (int e = 0; e < 16; ++e) {
+        const int row = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+        float sum = 0.f;
+        for (int k = 0; k < 16; ++k)
+            sum += as_float(g_ha[wave][s][row + 32 * (k / 8)][k % 8], 0, bf16) * as_float(g_hb[wave][s][col + 32 * (k / 8)][k % 8], 0, bf16);
+        acc16[e] += sum;
+    }
+}
+void host_mfma_32x32x2(float a_inst, float b_inst, float acc16[16]) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, s = t_slot32[1] ^= 1;
+    g_sa[wave][s][lane] = a_inst;
+    g_sb[wave][s][lane] = b_inst;
+    pthread_barrier_wait(&g_wave_barrier[wave]);
+    const int col = lane & 31;
+    for (int e = 0; e < 16; ++e) {
+        const int row = 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+        acc16[e] += g_sa[wave][s][row] * g_sb[wave][s][col] + g_sa[wave][s][row + 32] * g_sb[wave][s][col + 32];
+    }
+}
+
 namespace {
 using namespace sthip;
 
@@ -301,6 +333,90 @@ long run_case6(const char* name, int nprod, int M, int N, int K, bool sums, bool
     return bad_total;
 }
 
+// 256 x 128 kernel: classical (one segment, C = A B of M x N x K) or the seven segment products S_0..S_6 of
+// Mh x Nh x Kh recombined in registers into the four quadrants of C (2 Mh x 2 Nh), one accumulator tile parked
+// in global memory: Strassen order M3 M6 M5 M7 M1 M2 M4, Winograd order P1 P2 P6 P7 P5 P3 (-P4).
+template <class T, int ALGO, bool B_KC>
+long run_case3(const char* name, int Mh, int Nh, int Kh, bool out_f32, bool accumulate) {
+    constexpr bool bf = __is_same(T, bf16_t);
+    constexpr int NSEG = ALGO == ALGO_CLASSIC ? 1 : 7;
+    const int Q = ALGO == ALGO_CLASSIC ? 1 : 2;
+    const int es_out = out_f32 ? 4 : 2;
+    const size_t a_elems = (size_t)Mh * Kh, b_elems = (size_t)Kh * Nh, c_elems = (size_t)Q * Mh * Q * Nh;
+    const int ldc = Q * Nh;
+    std::vector<uint16_t> A(NSEG * a_elems), B(NSEG * b_elems);
+    std::vector<float> Af(NSEG * a_elems), Bf(NSEG * b_elems), C0(c_elems);
+    std::vector<char> C(c_elems * es_out);
+    uint32_t seed = 4242u + (uint32_t)(Mh + 5 * Nh + 11 * Kh + ALGO);
+    for (size_t i = 0; i < Af.size(); ++i) { Af[i] = (float)small_int(seed); A[i] = to_half(Af[i], bf); }
+    for (int p = 0; p < NSEG; ++p)
+        for (int k = 0; k < Kh; ++k)
+            for (int n = 0; n < Nh; ++n) {
+                const float v = (float)small_int(seed);
+                Bf[p * b_elems + (size_t)k * Nh + n] = v;
+                B[p * b_elems + (B_KC ? (size_t)n * Kh + k : (size_t)k * Nh + n)] = to_half(v, bf);
+            }
+    for (size_t i = 0; i < c_elems; ++i) {
+        C0[i] = accumulate ? (float)small_int(seed) : 0.f;
+        if (es_out == 4) memcpy(&C[i * 4], &C0[i], 4);
+        else { const uint16_t h = to_half(accumulate ? C0[i] : 77.f, bf); memcpy(&C[i * 2], &h, 2); }
+    }
+    g_global = {{reinterpret_cast<const char*>(A.data()), A.size() * 2}, {reinterpret_cast<const char*>(B.data()), B.size() * 2}};
+    Gemm2Params P;
+    memset(&P, 0, sizeof(P));
+    for (int p = 0; p < NSEG; ++p) P.seg[p] = Seg2{A.data() + p * a_elems, B.data() + p * b_elems, Kh, B_KC ? Kh : Nh, 0, 0};
+    P.c_rs = ldc; P.Mh = Mh; P.Nh = Nh; P.Kh = Kh; P.tiles_m = Mh / 256; P.tiles_n = Nh / 128; P.group_m = 4;
+    P.out_f32 = out_f32; P.accumulate = accumulate;
+    const unsigned grid = (unsigned)(P.tiles_m * P.tiles_n);
+    std::vector<float> park((size_t)grid * 256 * 128);
+    P.park = park.data();
+    // the segment products
+    std::vector<float> S(NSEG * (size_t)Mh * Nh, 0.f);
+    for (int p = 0; p < NSEG; ++p)
+        for (int m = 0; m < Mh; ++m)
+            for (int k = 0; k < Kh; ++k) {
+                const float a = Af[p * a_elems + (size_t)m * Kh + k];
+                if (a == 0.f) continue;
+                for (int n = 0; n < Nh; ++n) S[(p * (size_t)Mh + m) * Nh + n] += a * Bf[p * b_elems + (size_t)k * Nh + n];
+            }
+    auto seg = [&](int p, int m, int n) { return S[(p * (size_t)Mh + m) * Nh + n]; };
+    long bad_total = 0;
+    for (int late = 0; late < 2; ++late) {
+        g_late = late != 0;
+        std::vector<char> Cw = C;
+        P.C = Cw.data();
+        launch(gemm3_kernel<T, ALGO, B_KC>, P, grid, 256);
+        long bad = 0;
+        for (int m = 0; m < Q * Mh; ++m)
+            for (int n = 0; n < Q * Nh; ++n) {
+                const int qm = m / Mh, qn = n / Nh, mm = m % Mh, nn = n % Nh;
+                float want = C0[(size_t)m * ldc + n];
+                if (ALGO == ALGO_CLASSIC) want += seg(0, mm, nn);
+                else if (ALGO == ALGO_STRASSEN) {   // segments: 0 M3, 1 M6, 2 M5, 3 M7, 4 M1, 5 M2, 6 M4
+                    if (qm == 0 && qn == 0) want += seg(4, mm, nn) + seg(6, mm, nn) - seg(2, mm, nn) + seg(3, mm, nn);
+                    else if (qm == 0) want += seg(0, mm, nn) + seg(2, mm, nn);
+                    else if (qn == 0) want += seg(5, mm, nn) + seg(6, mm, nn);
+                    else want += seg(4, mm, nn) - seg(5, mm, nn) + seg(0, mm, nn) + seg(1, mm, nn);
+                } else {                            // segments: 0 P1, 1 P2, 2 P6, 3 P7, 4 P5, 5 P3, 6 -P4
+                    const float u2 = seg(0, mm, nn) + seg(2, mm, nn), u3 = u2 + seg(3, mm, nn);
+                    if (qm == 0 && qn == 0) want += seg(0, mm, nn) + seg(1, mm, nn);
+                    else if (qm == 0) want += u2 + seg(4, mm, nn) + seg(5, mm, nn);
+                    else if (qn == 0) want += u3 + seg(6, mm, nn);
+                    else want += u3 + seg(4, mm, nn);
+                }
+                float got;
+                const size_t i = (size_t)m * ldc + n;
+                if (es_out == 4) memcpy(&got, &Cw[i * 4], 4);
+                else { uint16_t h; memcpy(&h, &Cw[i * 2], 2); got = from_half(h, bf); }
+                if (got != want && bad++ < 5) fprintf(stderr, "  %s: C[%d][%d] = %g, expected %g\n", name, m, n, got, want);
+            }
+        printf("%s  loads %s: %ld wrong of %zu\n", name, late ? "at the last moment" : "at once", bad, c_elems);
+        fflush(stdout);
+        bad_total += bad;
+    }
+    return bad_total;
+}
+
 // Every tile id of a launch must map to a different (batch, product, tile row, tile column), all of them in range.
 long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int xcd_chunks, int group_m) {
     Gemm2Params P;
@@ -346,6 +462,11 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case6<true>("64x64 fp32, one product 128x128x64, B k-contiguous, accumulating", 1, 128, 128, 64, false, true);
     if (want()) bad += run_case6<false>("64x64 fp32, seven products 128x128x128 of operand sums, B n-contiguous", 7, 128, 128, 128, true, false);
     if (want()) bad += run_case6<true>("64x64 fp32, seven products 64x128x64 of operand sums, B k-contiguous", 7, 64, 128, 64, true, false);
+    // the 256 x 128 kernel: classical, and the seven products recombined in registers
+    if (want()) bad += run_case3<bf16_t, ALGO_CLASSIC, false>("256x128 bf16 classical, 256x256x192, B n-contiguous", 256, 256, 192, false, false);
+    if (want()) bad += run_case3<f16_t, ALGO_STRASSEN, false>("256x128 fp16 Strassen in registers, halves 256x128x128 -> fp32", 256, 128, 128, true, false);
+    if (want()) bad += run_case3<bf16_t, ALGO_STRASSEN, true>("256x128 bf16 Strassen in registers, halves 256x256x64, B k-contiguous, accumulating fp32", 256, 256, 64, true, true);
+    if (want()) bad += run_case3<bf16_t, ALGO_WINOGRAD, false>("256x128 bf16 Winograd in registers, halves 256x128x128 -> fp32", 256, 128, 128, true, false);
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
