@@ -417,6 +417,95 @@ long run_case3(const char* name, int Mh, int Nh, int Kh, bool out_f32, bool accu
     return bad_total;
 }
 
+// 128 x 128 pipelined kernel: `nprod` classical products side by side, or the seven segment products recombined in
+// registers (three accumulator tiles, nothing parked).  A may be stored k x m (m-contiguous).
+template <class T, int ALGO, bool A_KC, bool B_KC>
+long run_case2(const char* name, int nprod, int Mh, int Nh, int Kh, bool out_f32, bool accumulate) {
+    constexpr bool bf = __is_same(T, bf16_t);
+    const int NSEG = ALGO == ALGO_CLASSIC ? nprod : 7;
+    const int Q = ALGO == ALGO_CLASSIC ? 1 : 2;
+    const int es_out = out_f32 ? 4 : 2;
+    const size_t a_elems = (size_t)Mh * Kh, b_elems = (size_t)Kh * Nh, c_one = (size_t)Q * Mh * Q * Nh;
+    const size_t c_elems = (ALGO == ALGO_CLASSIC ? nprod : 1) * c_one;
+    const int ldc = Q * Nh;
+    std::vector<uint16_t> A(NSEG * a_elems), B(NSEG * b_elems);
+    std::vector<float> Af(NSEG * a_elems), Bf(NSEG * b_elems), C0(c_elems);
+    std::vector<char> C(c_elems * es_out);
+    uint32_t seed = 777u + (uint32_t)(Mh + 5 * Nh + 11 * Kh + ALGO + 2 * A_KC + B_KC);
+    for (int p = 0; p < NSEG; ++p) {
+        for (int m = 0; m < Mh; ++m)
+            for (int k = 0; k < Kh; ++k) {
+                const float v = (float)small_int(seed);
+                Af[p * a_elems + (size_t)m * Kh + k] = v;
+                A[p * a_elems + (A_KC ? (size_t)m * Kh + k : (size_t)k * Mh + m)] = to_half(v, bf);
+            }
+        for (int k = 0; k < Kh; ++k)
+            for (int n = 0; n < Nh; ++n) {
+                const float v = (float)small_int(seed);
+                Bf[p * b_elems + (size_t)k * Nh + n] = v;
+                B[p * b_elems + (B_KC ? (size_t)n * Kh + k : (size_t)k * Nh + n)] = to_half(v, bf);
+            }
+    }
+    for (size_t i = 0; i < c_elems; ++i) {
+        C0[i] = accumulate ? (float)small_int(seed) : 0.f;
+        if (es_out == 4) memcpy(&C[i * 4], &C0[i], 4);
+        else { const uint16_t h = to_half(accumulate ? C0[i] : 77.f, bf); memcpy(&C[i * 2], &h, 2); }
+    }
+    g_global = {{reinterpret_cast<const char*>(A.data()), A.size() * 2}, {reinterpret_cast<const char*>(B.data()), B.size() * 2}};
+    Gemm2Params P;
+    memset(&P, 0, sizeof(P));
+    for (int p = 0; p < NSEG; ++p) P.seg[p] = Seg2{A.data() + p * a_elems, B.data() + p * b_elems, A_KC ? Kh : Mh, B_KC ? Kh : Nh, 0, 0};
+    P.c_rs = ldc; P.c_ps = (int64_t)c_one; P.nprod = ALGO == ALGO_CLASSIC ? nprod : 0;
+    P.Mh = Mh; P.Nh = Nh; P.Kh = Kh; P.tiles_m = Mh / 128; P.tiles_n = Nh / 128; P.group_m = 4;
+    P.out_f32 = out_f32; P.accumulate = accumulate;
+    const unsigned grid = (unsigned)(P.tiles_m * P.tiles_n * (ALGO == ALGO_CLASSIC ? nprod : 1));
+    std::vector<float> S(NSEG * (size_t)Mh * Nh, 0.f);
+    for (int p = 0; p < NSEG; ++p)
+        for (int m = 0; m < Mh; ++m)
+            for (int k = 0; k < Kh; ++k) {
+                const float a = Af[p * a_elems + (size_t)m * Kh + k];
+                if (a == 0.f) continue;
+                for (int n = 0; n < Nh; ++n) S[(p * (size_t)Mh + m) * Nh + n] += a * Bf[p * b_elems + (size_t)k * Nh + n];
+            }
+    auto seg = [&](int p, int m, int n) { return S[(p * (size_t)Mh + m) * Nh + n]; };
+    long bad_total = 0;
+    for (int late = 0; late < 2; ++late) {
+        g_late = late != 0;
+        std::vector<char> Cw = C;
+        P.C = Cw.data();
+        launch(gemm2_kernel<T, ALGO, A_KC, B_KC>, P, grid, 256);
+        long bad = 0;
+        for (int q = 0; q < (ALGO == ALGO_CLASSIC ? nprod : 1); ++q)
+            for (int m = 0; m < Q * Mh; ++m)
+                for (int n = 0; n < Q * Nh; ++n) {
+                    const int qm = m / Mh, qn = n / Nh, mm = m % Mh, nn = n % Nh;
+                    const size_t i = q * c_one + (size_t)m * ldc + n;
+                    float want = C0[i];
+                    if (ALGO == ALGO_CLASSIC) want += seg(q, mm, nn);
+                    else if (ALGO == ALGO_STRASSEN) {
+                        if (qm == 0 && qn == 0) want += seg(4, mm, nn) + seg(6, mm, nn) - seg(2, mm, nn) + seg(3, mm, nn);
+                        else if (qm == 0) want += seg(0, mm, nn) + seg(2, mm, nn);
+                        else if (qn == 0) want += seg(5, mm, nn) + seg(6, mm, nn);
+                        else want += seg(4, mm, nn) - seg(5, mm, nn) + seg(0, mm, nn) + seg(1, mm, nn);
+                    } else {
+                        const float u2 = seg(0, mm, nn) + seg(2, mm, nn), u3 = u2 + seg(3, mm, nn);
+                        if (qm == 0 && qn == 0) want += seg(0, mm, nn) + seg(1, mm, nn);
+                        else if (qm == 0) want += u2 + seg(4, mm, nn) + seg(5, mm, nn);
+                        else if (qn == 0) want += u3 + seg(6, mm, nn);
+                        else want += u3 + seg(4, mm, nn);
+                    }
+                    float got;
+                    if (es_out == 4) memcpy(&got, &Cw[i * 4], 4);
+                    else { uint16_t h; memcpy(&h, &Cw[i * 2], 2); got = from_half(h, bf); }
+                    if (got != want && bad++ < 5) fprintf(stderr, "  %s: C[%d][%d][%d] = %g, expected %g\n", name, q, m, n, got, want);
+                }
+        printf("%s  loads %s: %ld wrong of %zu\n", name, late ? "at the last moment" : "at once", bad, c_elems);
+        fflush(stdout);
+        bad_total += bad;
+    }
+    return bad_total;
+}
+
 // Every tile id of a launch must map to a different (batch, product, tile row, tile column), all of them in range.
 long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int xcd_chunks, int group_m) {
     Gemm2Params P;
@@ -467,6 +556,11 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case3<f16_t, ALGO_STRASSEN, false>("256x128 fp16 Strassen in registers, halves 256x128x128 -> fp32", 256, 128, 128, true, false);
     if (want()) bad += run_case3<bf16_t, ALGO_STRASSEN, true>("256x128 bf16 Strassen in registers, halves 256x256x64, B k-contiguous, accumulating fp32", 256, 256, 64, true, true);
     if (want()) bad += run_case3<bf16_t, ALGO_WINOGRAD, false>("256x128 bf16 Winograd in registers, halves 256x128x128 -> fp32", 256, 128, 128, true, false);
+    // the 128 x 128 pipelined kernel
+    if (want()) bad += run_case2<bf16_t, ALGO_CLASSIC, true, false>("128x128 bf16, three products of 128x256x128 side by side", 3, 128, 256, 128, false, false);
+    if (want()) bad += run_case2<f16_t, ALGO_CLASSIC, false, true>("128x128 fp16, A m-contiguous, B k-contiguous, 256x128x192, accumulating", 1, 256, 128, 192, false, true);
+    if (want()) bad += run_case2<bf16_t, ALGO_STRASSEN, true, false>("128x128 bf16 Strassen in registers, halves 128x128x64, 16-bit result", 1, 128, 128, 64, false, false);
+    if (want()) bad += run_case2<f16_t, ALGO_WINOGRAD, false, false>("128x128 fp16 Winograd in registers, A m-contiguous, halves 128x256x128 -> fp32, accumulating", 1, 128, 256, 128, true, true);
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
