@@ -32,6 +32,8 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 struct bf16_t { uint16_t v; };   // tag types: storage is 2 bytes, arithmetic is explicit
 struct f16_t { uint16_t v; };
 
+__device__ s16x4 lds_read_tr16_b64(const char* p);   // the transposing LDS read, defined in sthip_prims.hpp
+
 enum { ALGO_CLASSIC = 0, ALGO_STRASSEN = 1, ALGO_WINOGRAD = 2 };
 
 // Everything the kernel needs, passed by value.  Strides are in elements.
@@ -274,9 +276,8 @@ __device__ __forceinline__ u32x4 read_frag(const char* tile, int sub, int kg) {
         const int k0 = kg * 16 + (grp >> 1) * 8 + (l16 >> 2);
         const int col = sub + (grp & 1) * 16 + (l16 & 3) * 4;
         const char* p = tile + k0 * G::ROWB + col * 2;
-        typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * G::ROWB));
+        s16x4 lo = lds_read_tr16_b64(p);
+        s16x4 hi = lds_read_tr16_b64(p + 4 * G::ROWB);
         u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
         u32x4 r = {a[0], a[1], b[0], b[1]};
         return r;

@@ -506,6 +506,77 @@ long run_case2(const char* name, int nprod, int Mh, int Nh, int Kh, bool out_f32
     return bad_total;
 }
 
+// The fused 128 x 128 kernel (operands straight from A and B, quadrant sums formed in registers, seven products
+// recombined in registers): C = A B over the whole M x N x K problem, any sizes with EDGE (virtual zero padding).
+template <class T, int ALGO, bool A_KC, bool B_KC, bool EDGE>
+long run_case_fused(const char* name, int M, int N, int K, bool out_f32, bool accumulate) {
+    constexpr bool f32 = __is_same(T, float), bf = __is_same(T, bf16_t);
+    constexpr int ES = f32 ? 4 : 2, EPC = 16 / ES;
+    const int es_out = (f32 || out_f32) ? 4 : 2;
+    std::vector<char> A((size_t)M * K * ES), B((size_t)K * N * ES), C((size_t)M * N * es_out);
+    std::vector<float> Af((size_t)M * K), Bf((size_t)K * N), C0((size_t)M * N);
+    uint32_t seed = 31337u + (uint32_t)(M + 5 * N + 11 * K + ALGO + 2 * A_KC + B_KC);
+    auto put = [&](std::vector<char>& buf, size_t i, float v) {
+        if (f32) memcpy(&buf[i * 4], &v, 4);
+        else { const uint16_t h = to_half(v, bf); memcpy(&buf[i * 2], &h, 2); }
+    };
+    for (int m = 0; m < M; ++m)
+        for (int k = 0; k < K; ++k) {
+            const float v = (float)small_int(seed);
+            Af[(size_t)m * K + k] = v;
+            put(A, A_KC ? (size_t)m * K + k : (size_t)k * M + m, v);
+        }
+    for (int k = 0; k < K; ++k)
+        for (int n = 0; n < N; ++n) {
+            const float v = (float)small_int(seed);
+            Bf[(size_t)k * N + n] = v;
+            put(B, B_KC ? (size_t)n * K + k : (size_t)k * N + n, v);
+        }
+    for (size_t i = 0; i < C0.size(); ++i) {
+        C0[i] = accumulate ? (float)small_int(seed) : 0.f;
+        if (es_out == 4) memcpy(&C[i * 4], &C0[i], 4);
+        else { const uint16_t h = to_half(accumulate ? C0[i] : 77.f, bf); memcpy(&C[i * 2], &h, 2); }
+    }
+    const bool split = ALGO != ALGO_CLASSIC;
+    GemmParams P;
+    memset(&P, 0, sizeof(P));
+    P.A = A.data(); P.B = B.data();
+    P.a_rs = A_KC ? K : 1; P.a_cs = A_KC ? 1 : M;
+    P.b_rs = B_KC ? 1 : N; P.b_cs = B_KC ? K : 1;
+    P.c_rs = N; P.c_cs = 1;
+    P.M = M; P.N = N; P.K = K;
+    P.Mh = split ? (M + 1) / 2 : M; P.Nh = split ? (N + 1) / 2 : N; P.Kh = split ? (K + 1) / 2 : K;
+    P.tiles_m = (P.Mh + 127) / 128; P.tiles_n = (P.Nh + 127) / 128;
+    P.out_f32 = es_out == 4 && !f32 ? 1 : (f32 ? 1 : 0); P.accumulate = accumulate; P.group_m = 8;
+    const int a_long = A_KC ? K : M, b_long = B_KC ? K : N, a_blk = A_KC ? P.Kh : P.Mh, b_blk = B_KC ? P.Kh : P.Nh;
+    P.a_vec = a_long % EPC == 0 && (!split || a_blk % EPC == 0);
+    P.b_vec = b_long % EPC == 0 && (!split || b_blk % EPC == 0);
+    P.c_vec = N % 4 == 0 && (!split || P.Nh % 4 == 0);
+    long bad_total = 0;
+    g_global.clear();
+    for (int late = 0; late < 1; ++late) {   // this kernel loads through registers with plain loads: one timing
+        g_late = false;
+        std::vector<char> Cw = C;
+        P.C = Cw.data();
+        launch(gemm_kernel<T, ALGO, A_KC, B_KC, EDGE>, P, (unsigned)(P.tiles_m * P.tiles_n), 256);
+        long bad = 0;
+        for (int m = 0; m < M; ++m)
+            for (int n = 0; n < N; ++n) {
+                float want = C0[(size_t)m * N + n];
+                for (int k = 0; k < K; ++k) want += Af[(size_t)m * K + k] * Bf[(size_t)k * N + n];
+                float got;
+                const size_t i = (size_t)m * N + n;
+                if (es_out == 4) memcpy(&got, &Cw[i * 4], 4);
+                else { uint16_t h; memcpy(&h, &Cw[i * 2], 2); got = from_half(h, bf); }
+                if (got != want && bad++ < 5) fprintf(stderr, "  %s: C[%d][%d] = %g, expected %g\n", name, m, n, got, want);
+            }
+        printf("%s: %ld wrong of %zu\n", name, bad, (size_t)M * N);
+        fflush(stdout);
+        bad_total += bad;
+    }
+    return bad_total;
+}
+
 // Every tile id of a launch must map to a different (batch, product, tile row, tile column), all of them in range.
 long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int xcd_chunks, int group_m) {
     Gemm2Params P;
@@ -561,6 +632,13 @@ int main(int argc, char** argv) {
     if (want()) bad += run_case2<f16_t, ALGO_CLASSIC, false, true>("128x128 fp16, A m-contiguous, B k-contiguous, 256x128x192, accumulating", 1, 256, 128, 192, false, true);
     if (want()) bad += run_case2<bf16_t, ALGO_STRASSEN, true, false>("128x128 bf16 Strassen in registers, halves 128x128x64, 16-bit result", 1, 128, 128, 64, false, false);
     if (want()) bad += run_case2<f16_t, ALGO_WINOGRAD, false, false>("128x128 fp16 Winograd in registers, A m-contiguous, halves 128x256x128 -> fp32, accumulating", 1, 128, 256, 128, true, true);
+    // the fused kernel: whole problems, quadrant sums in registers; odd sizes through the EDGE form
+    if (want()) bad += run_case_fused<bf16_t, ALGO_STRASSEN, true, false, false>("fused bf16 Strassen, 256x256x128", 256, 256, 128, false, false);
+    if (want()) bad += run_case_fused<f16_t, ALGO_WINOGRAD, true, true, false>("fused fp16 Winograd, B k-contiguous, 256x512x128 -> fp32, accumulating", 256, 512, 128, true, true);
+    if (want()) bad += run_case_fused<bf16_t, ALGO_STRASSEN, true, false, true>("fused bf16 Strassen, odd sizes 201x137x99", 201, 137, 99, false, false);
+    if (want()) bad += run_case_fused<f16_t, ALGO_WINOGRAD, false, true, true>("fused fp16 Winograd, A m-contiguous, B k-contiguous, odd sizes 130x260x77 -> fp32", 130, 260, 77, true, false);
+    if (want()) bad += run_case_fused<float, ALGO_STRASSEN, true, false, true>("fused fp32 Strassen, odd sizes 150x131x45, accumulating", 150, 131, 45, true, true);
+    if (want()) bad += run_case_fused<bf16_t, ALGO_CLASSIC, false, false, true>("fused bf16 classical, A m-contiguous, 129x257x65", 129, 257, 65, false, false);
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);

@@ -1,5 +1,6 @@
 """The 256 x 256 kernels of strassen-triton_amd/csrc/sthip_kernel4.hpp, the 256 x 128 and 128 x 128 pipelined
-kernels of sthip_kernel3.hpp / sthip_kernel2.hpp (classical, and Strassen / Winograd recombined in registers) and the 64 x 64 fp32 kernel of sthip_kernel6.hpp
+kernels of sthip_kernel3.hpp / sthip_kernel2.hpp (classical, and Strassen / Winograd recombined in registers), the
+fused kernel of sthip_kernel.hpp (whole problems C = A B with the quadrant sums formed in registers, odd sizes included) and the 64 x 64 fp32 kernel of sthip_kernel6.hpp
 compiled for the host and run on the CPU, one thread per lane (tests/host_model/kernel4_host.cpp).
 
 The kernel headers are the library's own; only their inline-assembly statements are taken out (scheduling
@@ -92,11 +93,16 @@ def test_strip_asm_takes_out_whole_statements():
 
 @needs_clang
 def test_kernels_exact_on_the_host(tmp_path):
-    exe = _build(str(tmp_path), "plain")
-    r = subprocess.run([exe], capture_output=True, text=True, timeout=900)
+    try:   # under AddressSanitizer where the compiler has it: operands, results and the parked tile are heap buffers
+        exe = _build(str(tmp_path), "asan", extra=("-g", "-fsanitize=address"))
+    except AssertionError:
+        exe = _build(str(tmp_path), "plain")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
+    assert "AddressSanitizer" not in r.stderr, r.stderr[:4000]
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
-    assert len(lines) == 57 and all(": 0 wrong of" in l for l in lines), r.stdout   # 24 launches x 2 load timings, 9 tile numberings
+    # 24 launches of the pipelined kernels x 2 load timings, 6 of the fused kernel, 9 tile numberings
+    assert len(lines) == 63 and all(": 0 wrong of" in l for l in lines), r.stdout
     assert "ALL EXACT" in r.stdout
 
 
