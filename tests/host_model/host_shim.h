@@ -66,3 +66,9 @@ template <class V> inline V __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float 
 // Used directly by the fused 128 x 128 kernel of sthip_kernel.hpp, which this build does not run.
 typedef short host_s16x4 __attribute__((ext_vector_type(4)));
 template <class P> inline host_s16x4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(P) { abort(); }
+
+// The one-launch kernel's counters (sthip_kernel5.hpp): workgroups of that launch would have to run at the
+// same time, which this build does not do; the code only has to compile.
+#define __HIP_MEMORY_SCOPE_AGENT 4
+inline void __builtin_amdgcn_s_sleep(int) {}
+inline void __builtin_amdgcn_fence(int, const char*) {}

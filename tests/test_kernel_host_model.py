@@ -77,7 +77,8 @@ def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp", extra=()):
         open(os.path.join(inc, h), "w").write(text)
     exe = os.path.join(inc, "kernel4_host")
     cmd = [_clang(), "-std=c++17", "-O1", "-Wno-everything", "-no-pie", "-pthread", *extra, "-I", inc, "-I", MODEL,
-           "-I", os.path.join(ROOT, "include"), os.path.join(MODEL, "kernel4_host.cpp"), "-o", exe]
+           "-I", os.path.join(ROOT, "include"), os.path.join(MODEL, "kernel4_host.cpp"), os.path.join(MODEL, "host_runtime.cpp"),
+           "-o", exe]
     r = subprocess.run(cmd, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     return exe
