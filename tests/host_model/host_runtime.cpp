@@ -195,15 +195,16 @@ void host_launch(dim3 grid, dim3 block, const std::function<void()>& body) {
     if (threads % kLanes != 0 || threads > kThreadsWg) { fprintf(stderr, "host_launch: block of %d threads\n", threads); _Exit(2); }
     pthread_barrier_destroy(&g_wg_barrier);
     pthread_barrier_init(&g_wg_barrier, nullptr, threads);
+    for (unsigned bz = 0; bz < grid.z; ++bz)
     for (unsigned by = 0; by < grid.y; ++by)
         for (unsigned bx = 0; bx < grid.x; ++bx) {
             std::vector<std::thread> th;
             th.reserve(threads);
             for (int t = 0; t < threads; ++t)
-                th.emplace_back([&, t, bx, by] {
+                th.emplace_back([&, t, bx, by, bz] {
                     threadIdx = {(unsigned)t, 0, 0};
-                    blockIdx = {bx, by, 0};
-                    gridDim = {grid.x, grid.y, 1};
+                    blockIdx = {bx, by, bz};
+                    gridDim = {grid.x, grid.y, grid.z};
                     blockDim = {(unsigned)threads, 1, 1};
                     t_pending.clear();
                     body();

@@ -84,6 +84,39 @@ def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp", extra=()):
     return exe
 
 
+def _build_library(tmp, name, extra=()):
+    """Every translation unit of the library (strassen-triton_amd/build.py lists them) compiled for the host against the
+    stand-in HIP runtime of tests/host_model/hip/hip_runtime.h, linked with library_host.cpp and host_runtime.cpp."""
+    import glob
+    import importlib.util
+    from concurrent.futures import ThreadPoolExecutor
+    out = os.path.join(tmp, name)
+    os.makedirs(out)
+    for f in glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(CSRC, "*.hip")):
+        if os.path.basename(f) == "sthip_prims.hpp":   # the host build has its own (tests/host_model/sthip_prims.hpp)
+            continue
+        open(os.path.join(out, os.path.basename(f)), "w").write(strip_asm(open(f).read()).replace("extern __shared__", "extern"))
+    spec = importlib.util.spec_from_file_location("sthip_build", os.path.join(ROOT, "strassen-triton_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    common = ["-std=c++17", "-O1", "-Wno-everything", "-pthread", *extra, "-I", MODEL, "-I", out, "-I", os.path.join(ROOT, "include")]
+
+    def compile_unit(unit):
+        obj, src, defs = unit
+        r = subprocess.run([_clang(), "-x", "c++", *common, *defs, "-c", os.path.join(out, src), "-o", os.path.join(out, obj)],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, obj + "\n" + r.stderr[-3000:]
+        return os.path.join(out, obj)
+
+    with ThreadPoolExecutor(8) as pool:
+        objs = list(pool.map(compile_unit, build._units()))
+    exe = os.path.join(out, "library_host")
+    r = subprocess.run([_clang(), *common, "-no-pie", os.path.join(MODEL, "library_host.cpp"), os.path.join(MODEL, "host_runtime.cpp"),
+                        *objs, "-o", exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    return exe
+
+
 needs_clang = pytest.mark.skipif(_clang() is None, reason="no clang++ (the kernel headers use ext_vector_type)")
 
 
@@ -119,6 +152,20 @@ def test_no_data_race_under_thread_sanitizer(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
     assert "ThreadSanitizer" not in r.stderr, r.stderr[:4000]
     assert r.returncode == 0 and "ALL EXACT" in r.stdout, r.stdout[-2000:]
+
+
+@needs_clang
+def test_library_through_its_c_abi_on_the_host(tmp_path):
+    """sthip_gemm itself, host code and kernels, on the CPU: the headline path (sums, grouped 256 x 256 products walked by
+    fewer workgroups than tiles, recombination) and the two-level path (49 products) bit for bit against the cast schedule
+    written out in library_host.cpp, fp32 results, the classical product, the 64 x 64 fp32 path, the fused kernel on odd
+    sizes, Winograd on grouped 128 x 128 tiles accumulating into fp32."""
+    exe = _build_library(str(tmp_path), "lib")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
+    assert len(lines) == 7 and all(": 0 wrong of" in l for l in lines), r.stdout
+    assert "ALL EXACT" in r.stdout
 
 
 def _drop_barrier(text):
