@@ -53,3 +53,10 @@ def force_tile():
     yield force
     if first:
         lib.sthip_debug_force_tile(names[first[0]])
+
+
+@pytest.fixture(scope="session")
+def host_builds(tmp_path_factory):
+    """The kernels and the library compiled for the host (tests/test_kernel_host_model.py says how): host_builds("asan") etc."""
+    from test_kernel_host_model import HostBuilds
+    return HostBuilds(str(tmp_path_factory.mktemp("host_model")))

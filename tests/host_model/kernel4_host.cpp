@@ -408,10 +408,12 @@ long check_tile_numbering(int tiles_m, int tiles_n, int nprod, int nbatch, int x
 }
 
 int main(int argc, char** argv) {
+    // no argument: every case; "5": case 5 alone; "1/3": the cases whose number leaves 1 when divided by 3
     const int which = argc > 1 ? atoi(argv[1]) : -1;
-    long bad = 0;
+    const int shares = argc > 1 && strchr(argv[1], '/') ? atoi(strchr(argv[1], '/') + 1) : 0;
     int id = 0;
-    auto want = [&]() { return which < 0 || which == id++; };
+    auto want = [&]() { const int i = id++; return shares ? i % shares == which : which < 0 || which == i; };
+    long bad = 0;
     // workgroups that walk their tiles: 4 tiles on 2 workgroups, odd number of k-steps
     if (want()) bad += run_case<bf16_t, false>("walking bf16, B n-contiguous, 512x512x192, 2 workgroups", 1, 512, 512, 192, 2, true, false, false);
     if (want()) bad += run_case<bf16_t, true>("walking bf16, B k-contiguous, 512x512x192, 2 workgroups", 1, 512, 512, 192, 2, true, false, false);
@@ -450,7 +452,7 @@ int main(int argc, char** argv) {
     // fp32 operands (k-steps of 32)
     if (want()) bad += run_case<float, false>("one tile per workgroup fp32, B n-contiguous, 256x256x96", 1, 256, 256, 96, 0, false, true, false);
     if (want()) bad += run_case<float, true>("one tile per workgroup fp32, B k-contiguous, accumulating, 256x256x64", 1, 256, 256, 64, 0, false, true, true);
-    if (which < 0) {
+    if (which < 0 || (shares && which == 0)) {
         // the launcher's choices: chunks for products of 32 / 64 / 128 tiles with tiles_m % 4 == 0 and >= 256 tiles in all
         bad += check_tile_numbering(16, 16, 7, 1, 0, 4);
         bad += check_tile_numbering(32, 32, 1, 1, 0, 8);

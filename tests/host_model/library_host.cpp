@@ -128,9 +128,11 @@ long run_gemm(const char* name, int M, int N, int K, int dt, int out_dt, int alg
 }  // namespace
 
 int main(int argc, char** argv) try {
+    // no argument: every case; "5": case 5 alone; "1/3": the cases whose number leaves 1 when divided by 3
     const int which = argc > 1 ? atoi(argv[1]) : -1;
+    const int shares = argc > 1 && strchr(argv[1], '/') ? atoi(strchr(argv[1], '/') + 1) : 0;
     int id = 0;
-    auto want = [&]() { return which < 0 || which == id++; };
+    auto want = [&]() { const int i = id++; return shares ? i % shares == which : which < 0 || which == i; };
     long bad = 0;
     g_host_compute_units = 4;   // seven tiles on four "CUs": the grouped launch walks its tiles
     if (want()) bad += run_gemm("one level bf16, sums / grouped 256x256 products / recombination, 512x512x256", 512, 512, 256, STHIP_BF16, STHIP_BF16,

@@ -84,7 +84,7 @@ def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp", extra=()):
     return exe
 
 
-def _build_library(tmp, name, extra=()):
+def _build_library(tmp, name, extra=(), drivers=("library_host.cpp",)):
     """Every translation unit of the library (strassen-triton_amd/build.py lists them) compiled for the host against the
     stand-in HIP runtime of tests/host_model/hip/hip_runtime.h, linked with library_host.cpp and host_runtime.cpp."""
     import glob
@@ -110,11 +110,24 @@ def _build_library(tmp, name, extra=()):
 
     with ThreadPoolExecutor(8) as pool:
         objs = list(pool.map(compile_unit, build._units()))
-    exe = os.path.join(out, "library_host")
-    r = subprocess.run([_clang(), *common, "-no-pie", os.path.join(MODEL, "library_host.cpp"), os.path.join(MODEL, "host_runtime.cpp"),
-                        *objs, "-o", exe], capture_output=True, text=True)
+    runtime = os.path.join(out, "host_runtime.o")
+    r = subprocess.run([_clang(), *common, "-c", os.path.join(MODEL, "host_runtime.cpp"), "-o", runtime], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
-    return exe
+    exes = {}
+    for driver in drivers:
+        exes[driver] = os.path.join(out, driver[:-4])
+        r = subprocess.run([_clang(), *common, "-no-pie", os.path.join(MODEL, driver), runtime, *objs, "-o", exes[driver]],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-3000:]
+    return exes
+
+
+def run_shares(exe, shares=4, timeout=1800):
+    """The driver's cases dealt to `shares` processes that run side by side (a launch spends much of its time in barriers);
+    returns the worst exit code and everything printed."""
+    procs = [subprocess.Popen([exe, "%d/%d" % (i, shares)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True) for i in range(shares)]
+    outs = [p.communicate(timeout=timeout) for p in procs]
+    return max(abs(p.returncode) for p in procs), "".join(o[0] for o in outs), "".join(o[1] for o in outs)
 
 
 needs_clang = pytest.mark.skipif(_clang() is None, reason="no clang++ (the kernel headers use ext_vector_type)")
@@ -126,46 +139,41 @@ def test_strip_asm_takes_out_whole_statements():
 
 
 @needs_clang
-def test_kernels_exact_on_the_host(tmp_path):
-    try:   # under AddressSanitizer where the compiler has it: operands, results and the parked tile are heap buffers
-        exe = _build(str(tmp_path), "asan", extra=("-g", "-fsanitize=address"))
-    except AssertionError:
-        exe = _build(str(tmp_path), "plain")
-    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
-    assert "AddressSanitizer" not in r.stderr, r.stderr[:4000]
-    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
-    lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
+def test_kernels_exact_on_the_host(host_builds):
+    # under AddressSanitizer where the compiler has it: operands, results and the parked tile are heap buffers
+    exe = host_builds("asan") if host_builds.ok("asan") else host_builds("plain")
+    rc, out, err = run_shares(exe)
+    assert "AddressSanitizer" not in err, err[:4000]
+    assert rc == 0, out[-2000:] + err[-2000:]
+    lines = [l for l in out.splitlines() if "wrong of" in l]
     # 24 launches of the pipelined kernels x 2 load timings, 6 of the fused kernel, 9 tile numberings
-    assert len(lines) == 63 and all(": 0 wrong of" in l for l in lines), r.stdout
-    assert "ALL EXACT" in r.stdout
+    assert len(lines) == 63 and all(": 0 wrong of" in l for l in lines), out
+    assert out.count("ALL EXACT") == 4
 
 
 @needs_clang
-def test_no_data_race_under_thread_sanitizer(tmp_path):
+def test_no_data_race_under_thread_sanitizer(host_builds):
     """Lanes are threads, barriers are barriers, a direct-to-LDS load is a write by the issuing thread: an LDS
     buffer that is overwritten while another wave may still read it, or read before its barrier, is a data
     race that ThreadSanitizer reports whatever the timing of this run was."""
-    try:
-        exe = _build(str(tmp_path), "tsan", extra=("-g", "-fsanitize=thread"))
-    except AssertionError as e:   # no ThreadSanitizer runtime with this compiler
-        pytest.skip(str(e)[-300:])
-    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
-    assert "ThreadSanitizer" not in r.stderr, r.stderr[:4000]
-    assert r.returncode == 0 and "ALL EXACT" in r.stdout, r.stdout[-2000:]
+    if not host_builds.ok("tsan"):   # no ThreadSanitizer runtime with this compiler
+        pytest.skip(host_builds.why("tsan")[-300:])
+    rc, out, err = run_shares(host_builds("tsan"))
+    assert "ThreadSanitizer" not in err, err[:4000]
+    assert rc == 0 and out.count("ALL EXACT") == 4, out[-2000:]
 
 
 @needs_clang
-def test_library_through_its_c_abi_on_the_host(tmp_path):
+def test_library_through_its_c_abi_on_the_host(host_builds):
     """sthip_gemm itself, host code and kernels, on the CPU: the headline path (sums, grouped 256 x 256 products walked by
     fewer workgroups than tiles, recombination) and the two-level path (49 products) bit for bit against the cast schedule
     written out in library_host.cpp, fp32 results, the classical product, the 64 x 64 fp32 path, the fused kernel on odd
     sizes, Winograd on grouped 128 x 128 tiles accumulating into fp32."""
-    exe = _build_library(str(tmp_path), "lib")
-    r = subprocess.run([exe], capture_output=True, text=True, timeout=1800)
-    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
-    lines = [l for l in r.stdout.splitlines() if "wrong of" in l]
-    assert len(lines) == 7 and all(": 0 wrong of" in l for l in lines), r.stdout
-    assert "ALL EXACT" in r.stdout
+    rc, out, err = run_shares(host_builds("library")["library_host.cpp"], shares=3)
+    assert rc == 0, out[-3000:] + err[-3000:]
+    lines = [l for l in out.splitlines() if "wrong of" in l]
+    assert len(lines) == 7 and all(": 0 wrong of" in l for l in lines), out
+    assert out.count("ALL EXACT") == 3
 
 
 def _drop_barrier(text):
@@ -175,12 +183,10 @@ def _drop_barrier(text):
 
 
 @needs_clang
-def test_thread_sanitizer_sees_a_missing_barrier(tmp_path):
-    try:
-        exe = _build(str(tmp_path), "tsan_broken", _drop_barrier, extra=("-g", "-fsanitize=thread"))
-    except AssertionError as e:
-        pytest.skip(str(e)[-300:])
-    r = subprocess.run([exe, "0"], capture_output=True, text=True, timeout=900)
+def test_thread_sanitizer_sees_a_missing_barrier(host_builds):
+    if not host_builds.ok("tsan_broken"):
+        pytest.skip(host_builds.why("tsan_broken")[-300:])
+    r = subprocess.run([host_builds("tsan_broken"), "0"], capture_output=True, text=True, timeout=900)
     assert "ThreadSanitizer: data race" in r.stderr
 
 
@@ -202,12 +208,47 @@ def _short_wait6(text):   # 64 x 64 kernel: one load of the older register set m
     return text.replace(old, "        wait_vmcnt_imm<kLoadsPerSet + 1>();\n", 1)
 
 
+BROKEN = {"no wait before the barrier": (_drop_wait, "sthip_kernel4.hpp", "0"),
+          "cursor moved before the last load": (_advance_too_early, "sthip_kernel4.hpp", "0"),
+          "64x64: wait one load short": (_short_wait6, "sthip_kernel6.hpp", "12")}
+
+
 @needs_clang
-@pytest.mark.parametrize("mutate, header, case", [(_drop_wait, "sthip_kernel4.hpp", "0"), (_advance_too_early, "sthip_kernel4.hpp", "0"),
-                                                  (_short_wait6, "sthip_kernel6.hpp", "12")],
-                         ids=["no wait before the barrier", "cursor moved before the last load", "64x64: wait one load short"])
-def test_broken_copies_are_caught(tmp_path, mutate, header, case):
-    exe = _build(str(tmp_path), "broken", mutate, header)
-    r = subprocess.run([exe, case], capture_output=True, text=True, timeout=600)   # one launch is enough
+@pytest.mark.parametrize("name", list(BROKEN))
+def test_broken_copies_are_caught(host_builds, name):
+    r = subprocess.run([host_builds(name), BROKEN[name][2]], capture_output=True, text=True, timeout=600)   # one launch is enough
     assert r.returncode != 0, r.stdout
     assert "MODEL VIOLATION" in r.stderr or "FAILED" in r.stdout
+
+
+class HostBuilds:
+    """Every host build these tests and tests/test_host_parity.py use, made side by side once per session."""
+
+    def __init__(self, tmp):
+        from concurrent.futures import ThreadPoolExecutor
+        jobs = {"asan": lambda: _build(tmp, "asan", extra=("-g", "-fsanitize=address")),
+                "tsan": lambda: _build(tmp, "tsan", extra=("-g", "-fsanitize=thread")),
+                "tsan_broken": lambda: _build(tmp, "tsan_broken", _drop_barrier, extra=("-g", "-fsanitize=thread")),
+                "library": lambda: _build_library(tmp, "lib", drivers=("library_host.cpp", "library_cli.cpp"))}
+        for name, (mutate, header, _) in BROKEN.items():
+            jobs[name] = lambda mutate=mutate, header=header, name=name: _build(tmp, "broken%d" % list(BROKEN).index(name), mutate, header)
+        self.tmp, self.done = tmp, {}
+        with ThreadPoolExecutor(4) as pool:
+            for name, fut in [(n, pool.submit(j)) for n, j in jobs.items()]:
+                try:
+                    self.done[name] = fut.result()
+                except AssertionError as e:
+                    self.done[name] = e
+
+    def ok(self, name):
+        return not isinstance(self.done[name], Exception)
+
+    def why(self, name):
+        return str(self.done[name])
+
+    def __call__(self, name):
+        if name == "plain" and name not in self.done:
+            self.done[name] = _build(self.tmp, "plain")
+        if not self.ok(name):
+            raise self.done[name]
+        return self.done[name]
