@@ -21,7 +21,8 @@ inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { retu
 int host_compute_units();   // how many workgroups the "device" is said to run at once
 inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = host_compute_units(); return hipSuccess; }
 #define HIP_SYMBOL(x) (&(x))
-template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; return hipSuccess; }
+void host_register_symbol(const void* p, size_t bytes);   // a __device__ array becomes memory that kernels may read
+template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; host_register_symbol(sym, sizeof(T)); return hipSuccess; }
 #define __align__(n) __attribute__((aligned(n)))
 
 void host_launch(dim3 grid, dim3 block, const std::function<void()>& body);

@@ -20,6 +20,8 @@ thread_local HostDim3 threadIdx, blockIdx, gridDim, blockDim;
 namespace sthip { alignas(1024) char smem[160 * 1024]; }
 
 std::vector<HostRange> g_host_global;
+static std::vector<HostRange> g_host_symbols;
+void host_register_symbol(const void* p, size_t bytes) { g_host_symbols.push_back({(const char*)p, bytes}); }
 bool g_host_late = false;
 int g_host_compute_units = 4;
 int host_compute_units() { return g_host_compute_units; }
@@ -41,6 +43,8 @@ const char* g_xp[kWaves][2][kLanes];
 }
 void check_global(const char* p) {
     for (const HostRange& r : g_host_global)
+        if (p >= r.p && p + 16 <= r.p + r.n) return;
+    for (const HostRange& r : g_host_symbols)
         if (p >= r.p && p + 16 <= r.p + r.n) return;
     die("direct-to-LDS load reads outside the operands", p);
 }

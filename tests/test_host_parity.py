@@ -8,7 +8,6 @@ cases, STHIP_HOST_FULL=1 in the environment runs the whole grid (five to six min
 """
 import ctypes
 import os
-import struct
 import subprocess
 
 import pytest
@@ -21,7 +20,6 @@ pytestmark = pytest.mark.skipif(_clang() is None, reason="no clang++ for the hos
 
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 ALGO = {"classic": 0, "strassen": 1, "winograd": 2}
-TILE = {None: 0, "128x128": 1, "256x128": 2, "128x128g": 3, "256x256": 4, "64x64": 5}
 TOL = {torch.float32: 1e-5, torch.float16: 2e-2, torch.bfloat16: 2e-2}
 FULL = bool(os.environ.get("STHIP_HOST_FULL"))
 BF, HF, SG = torch.bfloat16, torch.float16, torch.float32
@@ -39,11 +37,6 @@ def cli(host_builds, tmp_path_factory):
     return host_builds("library")["library_cli.cpp"], str(tmp_path_factory.mktemp("jobs"))
 
 
-def _storage_bytes(t):
-    s = t.untyped_storage()
-    return ctypes.string_at(s.data_ptr(), s.nbytes())
-
-
 def _strides3(t):
     assert t.storage_offset() == 0
     if t.dim() == 2:
@@ -51,23 +44,68 @@ def _strides3(t):
     return (t.stride(0), t.stride(1), t.stride(2))
 
 
-def host_gemm(cli, A, B, algo="strassen", levels=1, out_dtype=None, out=None, accumulate=False, workspace=True, tile=None, cus=4):
-    exe, tmp = cli
+class Script:
+    """Statements for tests/host_model/library_cli.cpp: tensors become buffers of "device" memory (their whole storage, so
+    views keep their strides), calls name them, results are read back into the tensors after run()."""
+
+    def __init__(self, cli):
+        self.exe, self.tmp = cli
+        self.lines, self.back, self.count = [], [], 0
+
+    def buf(self, t, back=False):
+        if t is None:
+            return "-"
+        name = "b%d" % self.count
+        self.count += 1
+        s = t.untyped_storage()
+        path = os.path.join(self.tmp, name + ".bin")
+        with open(path, "wb") as f:
+            f.write(ctypes.string_at(s.data_ptr(), s.nbytes()))
+        self.lines.append("buf %s %d %s" % (name, s.nbytes(), path))
+        if back:
+            self.back.append((name, t))
+        return name
+
+    def add(self, *words):
+        self.lines.append(" ".join(str(int(w)) if isinstance(w, bool) else str(w) for w in words))
+
+    def workspace(self, batch, M, N, K, dt, odt, algo, levels):
+        name = "w%d" % self.count
+        self.count += 1
+        self.add("wsbuf", name, batch, M, N, K, dt, odt, algo, levels)
+        return name
+
+    def run(self):
+        for name, _ in self.back:
+            self.add("save", name, os.path.join(self.tmp, name + ".out"))
+        path = os.path.join(self.tmp, "script.txt")
+        with open(path, "w") as f:
+            f.write("\n".join(self.lines) + "\n")
+        r = subprocess.run([self.exe, path], capture_output=True, text=True, timeout=900)
+        assert r.returncode == 0, r.stderr[-2000:]
+        for name, t in self.back:
+            data = open(os.path.join(self.tmp, name + ".out"), "rb").read()
+            ctypes.memmove(t.untyped_storage().data_ptr(), data, len(data))
+
+
+def host_gemm(cli, A, B, algo="strassen", levels=1, out_dtype=None, out=None, accumulate=False, workspace=True, tile=None, cus=4,
+              static=False):
+    """strassen_hip.gemm on the host build: C = A B (or C += A B) through sthip_gemm, or sthip_gemm_static."""
     batch = A.shape[0] if A.dim() == 3 else 1
     M, K = A.shape[-2:]
     N = B.shape[-1]
     out_dtype = out_dtype or (out.dtype if out is not None else A.dtype)
     C = out if out is not None else torch.full((batch, M, N) if A.dim() == 3 else (M, N), 99.0).to(out_dtype)
-    a, b, c = _storage_bytes(A), _storage_bytes(B), _storage_bytes(C)
-    hdr = struct.pack("<4q9q3q8i", batch, M, N, K, *_strides3(A), *_strides3(B), *_strides3(C), len(a), len(b), len(c),
-                      DT[A.dtype], DT[out_dtype], ALGO[algo], levels, int(accumulate), int(workspace), TILE[tile], cus)
-    job, res = os.path.join(tmp, "job.bin"), os.path.join(tmp, "out.bin")
-    with open(job, "wb") as f:
-        f.write(hdr + a + b + c)
-    r = subprocess.run([exe, job, res], capture_output=True, text=True, timeout=900)
-    assert r.returncode == 0, r.stderr[-2000:]
-    data = open(res, "rb").read()
-    ctypes.memmove(C.untyped_storage().data_ptr(), data, len(data))
+    sc = Script(cli)
+    sc.add("units", cus)
+    sc.add("tile", tile or "-")
+    args = [sc.buf(A), sc.buf(B), sc.buf(C, back=True), batch, M, N, K, *_strides3(A), *_strides3(B), *_strides3(C),
+            DT[A.dtype], DT[out_dtype], ALGO[algo], levels, accumulate]
+    if static:
+        sc.add("gemm_static", *args)
+    else:
+        sc.add("gemm", *args, sc.workspace(batch, M, N, K, DT[A.dtype], DT[out_dtype], ALGO[algo], levels) if workspace else "-")
+    sc.run()
     return C
 
 
@@ -163,3 +201,96 @@ def test_gaussian_against_the_oracle(cli, dtype, levels, shape, tile):
     want = O.strassen_general(A, B, levels=levels, base_dtype=dtype, fp32_agg=True)
     assert O.rel_fro(C.double(), want.double()) <= TOL[dtype]
     assert O.rel_fro(C.double(), A.double() @ B.double()) <= TOL[dtype]
+
+
+# ---- the other entry points of include/strassen_hip.h (tests/test_gpu_api.py, tests/test_zz_no_alloc.py on the GPU) ----
+
+def test_static_entry_point_on_two_calls_in_a_row(cli):
+    """sthip_gemm_static against sthip_gemm, bit for bit: a first call, a smaller one with two levels, the first again."""
+    A, B = _gauss((512, 256), 51, 1.0, BF), _gauss((256, 512), 52, 1 / 16, BF)
+    A2, B2 = _gauss((256, 192), 53, 1.0, BF), _gauss((192, 256), 54, 1 / 14, BF)
+    sc = Script(cli)
+    outs = []
+    for a, b, levels in ((A, B, 1), (A2, B2, 2), (A, B, 1)):
+        M, K, N = *a.shape, b.shape[1]
+        for static in (True, False):
+            c = torch.full((M, N), 7.0).to(BF)
+            outs.append(c)
+            args = [sc.buf(a), sc.buf(b), sc.buf(c, back=True), 1, M, N, K, *_strides3(a), *_strides3(b), *_strides3(c), DT[BF], DT[BF], 1, levels, 0]
+            sc.add("gemm_static" if static else "gemm", *args, *([] if static else [sc.workspace(1, M, N, K, DT[BF], DT[BF], 1, levels)]))
+    sc.run()
+    for i in (0, 2, 4):
+        assert torch.equal(outs[i], outs[i + 1])
+    assert torch.equal(outs[0], outs[4])
+    assert O.rel_fro(outs[0].double(), A.double() @ B.double()) <= 2e-2
+    assert O.rel_fro(outs[2].double(), A2.double() @ B2.double()) <= 2e-2
+
+
+def test_static_entry_point_refuses_what_does_not_fit(cli):
+    sc = Script(cli)      # two levels at 8192^3 bf16 need more than the 144 MiB buffer; nothing is launched, no operand is read
+    tiny = torch.zeros(64, dtype=BF)
+    sc.add("expect", -4)
+    sc.add("gemm_static", sc.buf(tiny), sc.buf(tiny), sc.buf(tiny), 1, 8192, 8192, 8192, 0, 8192, 1, 0, 8192, 1, 0, 8192, 1, DT[BF], DT[BF], 1, 2, 0)
+    sc.run()
+
+
+@pytest.mark.parametrize("dtype,n,levels", [(BF, 256, 1), (SG, 128, 2), (HF, 256, 2), (BF, 64, 3)])
+def test_n_layers_entry_point(cli, dtype, n, levels):
+    """sthip_strassen_matmul_n_layers: square operands, B a transposed view (test_gpu_api.py:43)."""
+    A, Bt = _ints((n, n), 61, -1, 1, dtype), _ints((n, n), 62, -1, 1, dtype)
+    C = torch.zeros(n, n, dtype=dtype)
+    sc = Script(cli)
+    sc.add("n_layers", sc.buf(A), sc.buf(Bt), sc.buf(C, back=True), n, n, 1, 1, n, DT[dtype], levels, sc.workspace(1, n, n, n, DT[dtype], DT[dtype], 1, levels))
+    sc.run()
+    assert torch.equal(C.double(), A.double() @ Bt.double().t())
+
+
+@pytest.mark.parametrize("algo,levels", [("strassen", 1), ("strassen", 2), ("classic", 0)])
+def test_run_accumulate_entry_point(cli, algo, levels):
+    """sthip_run_accumulate: C += A B with fp16 operands and an fp32 C, batched (the contract of the reference's launchers)."""
+    A, B = _ints((2, 128, 64), 71, -1, 1, HF), _ints((2, 64, 256), 72, -1, 1, HF)
+    C0 = _ints((2, 128, 256), 73, -3, 3, SG)
+    C = C0.clone()
+    sc = Script(cli)
+    sc.add("run_accumulate", sc.buf(A), sc.buf(B), sc.buf(C, back=True), 2, 128, 256, 64, DT[HF], DT[SG], ALGO[algo], levels,
+           sc.workspace(2, 128, 256, 64, DT[HF], DT[SG], ALGO[algo], levels))
+    sc.run()
+    assert torch.equal(C.double(), C0.double() + A.double() @ B.double())
+
+
+@pytest.mark.parametrize("dtype,rows,D,levels,bias", [(BF, 256, 256, 1, True), (HF, 100, 256, 1, True), (BF, 512, 512, 2, False), (SG, 77, 128, 1, True)])
+def test_linear_strassen_forward_entry_point(cli, dtype, rows, D, levels, bias):
+    """sthip_linear_strassen_forward: y = x W^T + bias with rows <= D (reference model/layers.py:246-274 pads x instead)."""
+    x, W = _ints((rows, D), 81, -1, 1, dtype), _ints((D, D), 82, -1, 1, dtype)
+    b = _ints((D,), 83, -2, 2, dtype) if bias else None
+    y = torch.zeros(rows, D, dtype=dtype)
+    sc = Script(cli)
+    sc.add("linear_strassen", sc.buf(x), sc.buf(W), sc.buf(b), sc.buf(y, back=True), rows, D, DT[dtype], levels,
+           sc.workspace(1, rows, D, D, DT[dtype], DT[dtype], 1, levels))
+    sc.run()
+    assert torch.equal(y.double(), x.double() @ W.double().t() + (b.double() if bias else 0))
+
+
+@pytest.mark.parametrize("dtype,levels,rows,d_in,d_out,bias", [(BF, 1, 256, 256, 512, True), (HF, 2, 512, 512, 512, False), (BF, -2, 200, 136, 72, True)])
+def test_linear_forward_and_prepared_sums_same_bits(cli, dtype, levels, rows, d_in, d_out, bias):
+    """sthip_linear_forward on a layer of any shape; where sums of the weight can be kept, the forward that reads them gives the
+    same bits, and does read them: with the sums of another weight it gives another result (test_gpu_api.py:264)."""
+    x, W = _gauss((rows, d_in), 91, 1.0, dtype), _gauss((d_out, d_in), 92, d_in ** -0.5, dtype)
+    b = _gauss((d_out,), 93, 1.0, dtype) if bias else None
+    ys = [torch.zeros(rows, d_out, dtype=dtype) for _ in range(3)]
+    sc = Script(cli)
+    bx, bw, bb = sc.buf(x), sc.buf(W), sc.buf(b)
+    ws = sc.workspace(1, rows, d_out, d_in, DT[dtype], DT[dtype], 1, abs(levels))
+    sc.add("linear", bx, bw, bb, sc.buf(ys[0], back=True), rows, d_in, d_out, DT[dtype], levels, ws)
+    if levels > 0:
+        other = sc.buf(W.flip(0).contiguous())
+        for w_for_sums, y in ((bw, ys[1]), (other, ys[2])):
+            sc.add("sumsbuf", "sums", d_in, d_out, DT[dtype], levels)
+            sc.add("prepare", w_for_sums, d_in, d_out, DT[dtype], levels, "sums")
+            sc.add("linear_prepared", bx, bw, "sums", bb, sc.buf(y, back=True), rows, d_in, d_out, DT[dtype], levels, ws)
+    sc.run()
+    want = x.double() @ W.double().t() + (b.double() if bias else 0)
+    assert O.rel_fro(ys[0].double(), want) <= TOL[dtype]
+    if levels > 0:
+        assert torch.equal(ys[1], ys[0])
+        assert not torch.equal(ys[2], ys[0])
