@@ -7,7 +7,7 @@
 //   expect CODE               the following call must return CODE (default 0)
 //   gemm / gemm_static / n_layers / run_accumulate / linear_strassen / linear / prepare / linear_prepared ARGS...
 //                             the entry point of include/strassen_hip.h of that name, arguments in its order, buffers by
-//                             name ("-" = null), a workspace as one buffer name standing for pointer and size
+//                             name ("-" = null, NAME+BYTES = a view that starts BYTES into the buffer), a workspace as one buffer name standing for pointer and size
 #include <fstream>
 #include <map>
 #include <sstream>
@@ -26,7 +26,16 @@ static Buf* buf(std::istringstream& in) {
     if (!g_bufs.count(name)) { fprintf(stderr, "no buffer %s\n", name.c_str()); exit(2); }
     return &g_bufs[name];
 }
-static void* ptr(std::istringstream& in) { Buf* b = buf(in); return b ? b->p : nullptr; }
+static void* ptr(std::istringstream& in) {   // NAME or NAME+BYTES (a view that starts inside the buffer)
+    std::string name;
+    in >> name;
+    if (name == "-") return nullptr;
+    const size_t plus = name.find('+');
+    const size_t off = plus == std::string::npos ? 0 : std::stoull(name.substr(plus + 1));
+    name = name.substr(0, plus);
+    if (!g_bufs.count(name)) { fprintf(stderr, "no buffer %s\n", name.c_str()); exit(2); }
+    return g_bufs[name].p + off;
+}
 static int64_t num(std::istringstream& in) { long long v; if (!(in >> v)) { fprintf(stderr, "number expected\n"); exit(2); } return v; }
 static void strides(std::istringstream& in, int64_t s[3]) { for (int i = 0; i < 3; ++i) s[i] = num(in); }
 

@@ -38,7 +38,6 @@ def cli(host_builds, tmp_path_factory):
 
 
 def _strides3(t):
-    assert t.storage_offset() == 0
     if t.dim() == 2:
         return (0, t.stride(0), t.stride(1))
     return (t.stride(0), t.stride(1), t.stride(2))
@@ -64,7 +63,8 @@ class Script:
         self.lines.append("buf %s %d %s" % (name, s.nbytes(), path))
         if back:
             self.back.append((name, t))
-        return name
+        off = t.storage_offset() * t.element_size()
+        return name + "+%d" % off if off else name
 
     def add(self, *words):
         self.lines.append(" ".join(str(int(w)) if isinstance(w, bool) else str(w) for w in words))
@@ -201,6 +201,55 @@ def test_gaussian_against_the_oracle(cli, dtype, levels, shape, tile):
     want = O.strassen_general(A, B, levels=levels, base_dtype=dtype, fp32_agg=True)
     assert O.rel_fro(C.double(), want.double()) <= TOL[dtype]
     assert O.rel_fro(C.double(), A.double() @ B.double()) <= TOL[dtype]
+
+
+
+def _random_call(case):
+    """A seeded random sthip_gemm call: sizes aligned to tiles, to 8, or arbitrary; either layout of A and B; leading dimensions
+    with padding; views that start 2 or 16 bytes into their storage; batch; fp32 or native result; accumulate; with and without
+    workspace; a forced tile; 1 .. 16 compute units."""
+    import random
+    rnd = random.Random(1000 + case)
+    dt = rnd.choice([BF, BF, HF, SG])
+    algo = rnd.choice(["classic", "strassen", "strassen", "winograd"])
+    levels = 0 if algo == "classic" else rnd.choice([1, 1, 1, 2])
+    kind = rnd.random()
+    if kind < 0.35:
+        M, N, K = (rnd.choice([64, 128]) * rnd.randint(1, 3) for _ in range(3))
+    elif kind < 0.65:
+        M, N, K = (8 * rnd.randint(1, 30) for _ in range(3))
+    else:
+        M, N, K = (rnd.randint(1, 200) for _ in range(3))
+    if dt == SG:
+        K = min(K, 96)
+    batch = rnd.choice([0, 0, 0, 2])
+    opts = dict(algo=algo, levels=levels, accumulate=rnd.random() < 0.3, workspace=rnd.random() < 0.8 or levels >= 2,
+                tile=rnd.choice([None, None, None, "128x128", "128x128g", "256x128", "256x256", "64x64"]), cus=rnd.choice([1, 2, 4, 8, 16]))
+    g = torch.Generator().manual_seed(case)
+
+    def make(rows, cols, transposed, dtype, lo, hi):
+        pad, off = rnd.choice([0, 0, 8, 3]), rnd.choice([0, 0, 0, 8, 1])
+        r, c = (cols, rows) if transposed else (rows, cols)
+        flat = torch.randint(lo, hi + 1, (off + (batch or 1) * r * (c + pad),), generator=g).to(dtype)
+        v = flat[off:].view(*((batch,) if batch else ()), r, c + pad)[..., :c]
+        return v.transpose(-1, -2) if transposed else v
+
+    A = make(M, K, rnd.random() < 0.4, dt, -1, 1)
+    B = make(K, N, rnd.random() < 0.5, dt, -1, 1)
+    C = make(M, N, False, rnd.choice([dt, SG]), -3, 3)
+    return A, B, C, opts
+
+
+@pytest.mark.parametrize("case", range(_grid(200, 24)))
+def test_random_calls_exact(cli, case):
+    A, B, C, opts = _random_call(case)
+    C0, around = C.clone(), C._base.clone()
+    host_gemm(cli, A, B, out=C, **opts)
+    assert torch.equal(C.double(), A.double() @ B.double() + (C0.double() if opts["accumulate"] else 0)), opts
+    after = C._base.clone()     # nothing outside the view of C (padding of its rows, the elements in front of it) was written
+    for whole in (around, after):
+        whole.as_strided(C.size(), C.stride(), C.storage_offset()).zero_()
+    assert torch.equal(around, after), opts
 
 
 # ---- the other entry points of include/strassen_hip.h (tests/test_gpu_api.py, tests/test_zz_no_alloc.py on the GPU) ----
