@@ -10,6 +10,7 @@ stream, and the grid is limited by --max-n.
 
     python main_profiling.py [--dtype bf16|fp16|fp32] [--max-n 16384] [--min-n 1024]
     python main_profiling.py --gpt2      # the Linear shapes of GPT-2 small, forward and backward
+    python main_profiling.py --cutoff    # classical kernel against 1 - 3 Strassen levels: the measurement behind sthip_auto_levels
     python main_profiling.py --json out.json   # also write the rows as JSON
     python main_profiling.py --cache-weight-sums   # LinearStrassen keeps the weight's quadrant sums between calls
 """
@@ -165,12 +166,64 @@ def profile_gpt2_linears(tokens: int = 8192, dtype=torch.bfloat16) -> list[dict]
     return rows
 
 
+# M x N x K of the cutoff table: the square sizes around which a level starts to pay, and some that are not square.
+_CUTOFF_SHAPES = [(4096, 4096, 4096), (8192, 8192, 8192), (12288, 12288, 12288), (16384, 16384, 16384), (8192, 16384, 16384),
+                  (16384, 8192, 16384), (20480, 20480, 20480), (24576, 24576, 24576), (32768, 32768, 32768)]
+
+
+def _steady(fn, runs: int) -> float:
+    """Milliseconds per call of `runs` calls back to back (the state of a training or serving loop: operands of the next call
+    partly in the last-level cache, clocks settled), after a quarter as many warm-up calls."""
+    for _ in range(max(3, runs // 4)):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(runs):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / runs
+
+
+@torch.no_grad()
+def profile_cutoff(dtype=torch.bfloat16, shapes=None, max_levels: int = 2, b_transposed: bool = False, runs=None) -> list[dict]:
+    """The library's classical kernel against 1 .. max_levels Strassen levels on C = A B, beside torch.matmul and what
+    strassen_hip.auto_levels picks for the shape: the table from which the rule of sthip_auto_levels is read (a level pays
+    where its column is below the classical one).  The reference has no such cutoff; its replace_linear_with_strassen takes
+    every layer of at least min_size features (model/layers.py:279-300)."""
+    import strassen_hip
+    rows = []
+    print(f"{'M x N x K':>20s} | {'matmul ms':>9s} | {'classic ms':>10s} | " +
+          " | ".join(f"{f'{l} level ms':>10s}" for l in range(1, max_levels + 1)) + f" | {'best':>4s} | {'rule':>4s}")
+    for M, N, K in shapes or _CUTOFF_SHAPES:
+        a = torch.randn(M, K, device="cuda", dtype=dtype) * K ** -0.5
+        b = torch.randn(N, K, device="cuda", dtype=dtype).t() if b_transposed else torch.randn(K, N, device="cuda", dtype=dtype)
+        out = torch.empty(M, N, device="cuda", dtype=dtype)
+        n = runs or (30 if 2.0 * M * N * K <= 1e13 else 8)
+        r = dict(M=M, N=N, K=K, b_transposed=b_transposed, std_ms=_steady(lambda: torch.matmul(a, b, out=out), n))
+        r["level_ms"] = [_steady(lambda: strassen_hip.gemm(a, b, out, algo="classic", levels=0), n)]
+        for levels in range(1, max_levels + 1):
+            ws = torch.empty(max(1, strassen_hip.workspace_bytes(a, b, levels=levels)), dtype=torch.uint8, device="cuda")
+            r["level_ms"].append(_steady(lambda: strassen_hip.gemm(a, b, out, levels=levels, workspace=ws), n))
+            del ws
+        r["best_levels"] = min(range(max_levels + 1), key=lambda l: r["level_ms"][l])
+        r["rule_levels"] = strassen_hip.auto_levels(M, N, K, dtype, max_levels)
+        rows.append(r)
+        print(f"{f'{M}x{N}x{K}':>20s} | {r['std_ms']:>9.4f} | " + " | ".join(f"{t:>10.4f}" for t in r["level_ms"]) +
+              f" | {r['best_levels']:>4d} | {r['rule_levels']:>4d}", flush=True)
+        del a, b, out
+        torch.cuda.empty_cache()
+    return rows
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--dtype", choices=sorted(_DTYPES), default="bf16")
     ap.add_argument("--min-n", type=int, default=1024)
     ap.add_argument("--max-n", type=int, default=16384)
     ap.add_argument("--gpt2", action="store_true", help="GPT-2-small Linear shapes instead of the square grid")
+    ap.add_argument("--cutoff", action="store_true", help="classical kernel against Strassen levels on a grid of shapes up to --max-n")
+    ap.add_argument("--b-transposed", action="store_true", help="--cutoff: B as the transposed view of an N x K matrix (the layout of x W^T)")
     ap.add_argument("--cache-weight-sums", action="store_true",
                     help="keep the quadrant sums of the weight between calls (16-bit weights)")
     ap.add_argument("--json", default=None, help="write the measured rows to this file as JSON")
@@ -180,6 +233,9 @@ if __name__ == "__main__":
     print(f"device: {torch.cuda.get_device_name(0)}  dtype: {args.dtype}")
     if args.gpt2:
         rows = profile_gpt2_linears(dtype=_DTYPES[args.dtype])
+    elif args.cutoff:
+        rows = profile_cutoff(_DTYPES[args.dtype], [s for s in _CUTOFF_SHAPES if args.min_n <= max(s) <= args.max_n],
+                              max_levels=3 if args.max_n > 16384 else 2, b_transposed=args.b_transposed)
     else:
         rows = profile_linear_layers(_DTYPES[args.dtype], args.min_n, args.max_n, args.cache_weight_sums)
     if args.json:
