@@ -26,6 +26,15 @@ BF, HF, SG = torch.bfloat16, torch.float16, torch.float32
 ALGOS = ["classic", "strassen", "winograd"]
 
 
+def _name(v):
+    """Readable test ids: bf16, 512x256x384, NT ..."""
+    if isinstance(v, torch.dtype):
+        return {BF: "bf16", HF: "fp16", SG: "fp32"}[v]
+    if isinstance(v, tuple):
+        return "x".join(str(x) for x in v)
+    return None
+
+
 def _grid(full, short):
     """The whole grid of cases, or the part of it that the default run keeps."""
     return full if FULL else short
@@ -130,7 +139,7 @@ KAT = _grid([(d, a, *s) for d in (BF, HF, SG) for a in ALGOS for s in KAT_SHAPES
             [(d, a, *s) for d in (HF, SG) for a in ("strassen", "winograd") for s in KAT_SHAPES[:3]] + [(SG, "classic", *KAT_SHAPES[1])])
 
 
-@pytest.mark.parametrize("dtype,algo,ta,tb,shape", KAT)
+@pytest.mark.parametrize("dtype,algo,ta,tb,shape", KAT, ids=_name)
 def test_integer_kat_exact(cli, dtype, algo, ta, tb, shape):
     """Entries in [-2, 2]: the fp32 result must equal the fp64 classical product bit for bit (test_gpu_parity.py:65)."""
     M, N, K = shape
@@ -141,7 +150,7 @@ def test_integer_kat_exact(cli, dtype, algo, ta, tb, shape):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("algo", ["classic", "strassen", "winograd"])
-@pytest.mark.parametrize("shape", [(256, 256, 128), (96, 40, 100)])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (96, 40, 100)], ids=_name)
 def test_integer_kat_exact_native_output(cli, dtype, algo, shape):
     M, N, K = shape
     A, B = _ints((M, K), 3, -1, 1, dtype), _ints((K, N), 4, -1, 1, dtype)
@@ -153,7 +162,7 @@ DEEP = _grid([(d, l, s) for d in (BF, SG) for l, s in [(2, (512, 512, 512)), (2,
              [(BF, 2, (512, 512, 512)), (BF, 2, (67, 35, 129)), (BF, 3, (256, 256, 256)), (HF, 2, (256, 320, 192)), (SG, 2, (67, 35, 129))])
 
 
-@pytest.mark.parametrize("dtype,levels,shape", DEEP)
+@pytest.mark.parametrize("dtype,levels,shape", DEEP, ids=_name)
 def test_integer_kat_multi_level(cli, dtype, levels, shape):
     M, N, K = shape
     A, B = _ints((M, K), 5, -1, 1, dtype), _ints((K, N), 6, -1, 1, dtype)
@@ -179,7 +188,7 @@ TILE_CASES = _grid([(t, d, a) for t in TILES for d in (BF, HF) for a in ALGOS],
                    [("128x128g", HF, "winograd")])
 
 
-@pytest.mark.parametrize("tile,dtype,algo", TILE_CASES)
+@pytest.mark.parametrize("tile,dtype,algo", TILE_CASES, ids=_name)
 def test_every_pipelined_tile_exact(cli, tile, dtype, algo):
     """Every tile of the pipelined paths, forced, on a problem it fits (test_gpu_parity.py:389)."""
     M, N, K = 512, 512, 256
@@ -192,7 +201,7 @@ GAUSS_SHAPES = [(1, (512, 512, 256), "256x256"), (1, (384, 256, 320), None), (2,
 GAUSS = _grid([(d, *g) for d in (BF, HF, SG) for g in GAUSS_SHAPES], [(d, *g) for d in (BF, HF) for g in GAUSS_SHAPES] + [(SG, *GAUSS_SHAPES[1])])
 
 
-@pytest.mark.parametrize("dtype,levels,shape,tile", GAUSS)
+@pytest.mark.parametrize("dtype,levels,shape,tile", GAUSS, ids=_name)
 def test_gaussian_against_the_oracle(cli, dtype, levels, shape, tile):
     """N(0, 1/K) inputs against the oracle's recursion with fp32 aggregation, the tolerances of test_gpu_parity.py."""
     M, N, K = shape
@@ -283,7 +292,7 @@ def test_static_entry_point_refuses_what_does_not_fit(cli):
     sc.run()
 
 
-@pytest.mark.parametrize("dtype,n,levels", [(BF, 256, 1), (SG, 128, 2), (HF, 256, 2), (BF, 64, 3)])
+@pytest.mark.parametrize("dtype,n,levels", [(BF, 256, 1), (SG, 128, 2), (HF, 256, 2), (BF, 64, 3)], ids=_name)
 def test_n_layers_entry_point(cli, dtype, n, levels):
     """sthip_strassen_matmul_n_layers: square operands, B a transposed view (test_gpu_api.py:43)."""
     A, Bt = _ints((n, n), 61, -1, 1, dtype), _ints((n, n), 62, -1, 1, dtype)
@@ -294,7 +303,7 @@ def test_n_layers_entry_point(cli, dtype, n, levels):
     assert torch.equal(C.double(), A.double() @ Bt.double().t())
 
 
-@pytest.mark.parametrize("algo,levels", [("strassen", 1), ("strassen", 2), ("classic", 0)])
+@pytest.mark.parametrize("algo,levels", [("strassen", 1), ("strassen", 2), ("classic", 0)], ids=_name)
 def test_run_accumulate_entry_point(cli, algo, levels):
     """sthip_run_accumulate: C += A B with fp16 operands and an fp32 C, batched (the contract of the reference's launchers)."""
     A, B = _ints((2, 128, 64), 71, -1, 1, HF), _ints((2, 64, 256), 72, -1, 1, HF)
@@ -307,7 +316,7 @@ def test_run_accumulate_entry_point(cli, algo, levels):
     assert torch.equal(C.double(), C0.double() + A.double() @ B.double())
 
 
-@pytest.mark.parametrize("dtype,rows,D,levels,bias", [(BF, 256, 256, 1, True), (HF, 100, 256, 1, True), (BF, 512, 512, 2, False), (SG, 77, 128, 1, True)])
+@pytest.mark.parametrize("dtype,rows,D,levels,bias", [(BF, 256, 256, 1, True), (HF, 100, 256, 1, True), (BF, 512, 512, 2, False), (SG, 77, 128, 1, True)], ids=_name)
 def test_linear_strassen_forward_entry_point(cli, dtype, rows, D, levels, bias):
     """sthip_linear_strassen_forward: y = x W^T + bias with rows <= D (reference model/layers.py:246-274 pads x instead)."""
     x, W = _ints((rows, D), 81, -1, 1, dtype), _ints((D, D), 82, -1, 1, dtype)
@@ -320,7 +329,7 @@ def test_linear_strassen_forward_entry_point(cli, dtype, rows, D, levels, bias):
     assert torch.equal(y.double(), x.double() @ W.double().t() + (b.double() if bias else 0))
 
 
-@pytest.mark.parametrize("dtype,levels,rows,d_in,d_out,bias", [(BF, 1, 256, 256, 512, True), (HF, 2, 512, 512, 512, False), (BF, -2, 200, 136, 72, True)])
+@pytest.mark.parametrize("dtype,levels,rows,d_in,d_out,bias", [(BF, 1, 256, 256, 512, True), (HF, 2, 512, 512, 512, False), (BF, -2, 200, 136, 72, True)], ids=_name)
 def test_linear_forward_and_prepared_sums_same_bits(cli, dtype, levels, rows, d_in, d_out, bias):
     """sthip_linear_forward on a layer of any shape; where sums of the weight can be kept, the forward that reads them gives the
     same bits, and does read them: with the sums of another weight it gives another result (test_gpu_api.py:264)."""
