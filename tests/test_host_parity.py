@@ -217,6 +217,8 @@ def test_gaussian_against_the_oracle(cli, dtype, levels, shape, tile):
     (BF, (512, 512, 256), 1, BF, "256x256"),    # recombination pass adds into a 16-bit C
     (HF, (512, 512, 256), 1, SG, "256x256"),    # products kept in fp32, recombination adds into an fp32 C
     (BF, (256, 256, 128), 1, BF, "128x128g"),
+    (HF, (512, 256, 128), 1, HF, "256x128"),    # recombined in registers around the parked tile, added into a 16-bit C
+    (HF, (33, 17, 65), 1, HF, None),            # fused kernel, edge tiles, element-wise read-modify-write
     (BF, (132, 100, 72), 2, BF, None),          # two levels by host recursion, 16-bit C
     (SG, (256, 256, 128), 1, SG, "256x128"),    # fp32: sums written once, the seven products as one batched launch
     (SG, (128, 192, 64), 1, SG, "64x64")], ids=_name)
