@@ -4,6 +4,7 @@
 //   sumsbuf NAME in_features out_features dtype levels          a buffer of sthip_linear_weight_sums_bytes(...) bytes
 //   save NAME FILE            write a buffer to FILE
 //   units N                   compute units the "device" reports        tile NAME|-    force a tile of the pipelined paths
+//   stages MASK               sthip_debug_set_stages(MASK)
 //   expect CODE               the following call must return CODE (default 0)
 //   gemm / gemm_static / n_layers / run_accumulate / linear_strassen / linear / prepare / linear_prepared ARGS...
 //                             the entry point of include/strassen_hip.h of that name, arguments in its order, buffers by
@@ -93,6 +94,9 @@ int main(int argc, char** argv) {
             std::string t;
             in >> t;
             sthip_debug_force_tile(t == "-" ? nullptr : t.c_str());
+            call = false;
+        } else if (op == "stages") {
+            sthip_debug_set_stages((int)num(in));
             call = false;
         } else if (op == "expect") {
             expect = (int)num(in);

@@ -263,6 +263,38 @@ def test_paths_that_only_large_problems_take(cli, algo, levels, dtype, shape):
     assert torch.equal(C.double(), A.double() @ B.double())
 
 
+@pytest.mark.parametrize("stages", _grid([47, 31], [47]))
+def test_other_launch_forms_give_the_same_bits(cli, stages):
+    """The 256 x 256 kernel with one workgroup per tile instead of workgroups that walk their tiles (stage bit 5), and the
+    whole level as ONE launch whose workgroups are sums, product tiles and recombination ordered by counters (bit 4; the host
+    runs the workgroups one after the other in launch order, which is the order the counters assume)."""
+    A, B = _gauss((512, 256), 131, 1.0, BF), _gauss((256, 512), 132, 1 / 16, BF)
+    outs = []
+    for mask in (15, stages):
+        C = torch.zeros(512, 512, dtype=BF)
+        sc = Script(cli)
+        sc.add("tile", "256x256")
+        sc.add("stages", mask)
+        sc.add("gemm", sc.buf(A), sc.buf(B), sc.buf(C, back=True), 1, 512, 512, 256, *_strides3(A), *_strides3(B), *_strides3(C),
+               DT[BF], DT[BF], 1, 1, 0, sc.workspace(1, 512, 512, 256, DT[BF], DT[BF], 1, 1))
+        sc.run()
+        outs.append(C)
+    assert torch.equal(outs[0], outs[1])
+    assert O.rel_fro(outs[0].double(), A.double() @ B.double()) <= 2e-2
+
+
+def test_two_levels_by_host_recursion(cli):
+    """Stage bit 3 cleared: two levels never run as one 49-product launch but as seven one-level calls with fp32 results."""
+    A, B = _ints((512, 512), 141, -1, 1, BF), _ints((512, 256), 142, -1, 1, BF)
+    C = torch.zeros(512, 256, dtype=SG)
+    sc = Script(cli)
+    sc.add("stages", 7)
+    sc.add("gemm", sc.buf(A), sc.buf(B), sc.buf(C, back=True), 1, 512, 256, 512, *_strides3(A), *_strides3(B), *_strides3(C),
+           DT[BF], DT[SG], 1, 2, 0, sc.workspace(1, 512, 256, 512, DT[BF], DT[SG], 1, 2))
+    sc.run()
+    assert torch.equal(C.double(), A.double() @ B.double())
+
+
 def _random_call(case):
     """A seeded random sthip_gemm call: sizes aligned to tiles, to 8, or arbitrary; either layout of A and B; leading dimensions
     with padding; views that start 2 or 16 bytes into their storage; batch; fp32 or native result; accumulate; with and without
