@@ -140,10 +140,11 @@ def test_strip_asm_takes_out_whole_statements():
 
 @needs_clang
 def test_kernels_exact_on_the_host(host_builds):
-    # under AddressSanitizer where the compiler has it: operands, results and the parked tile are heap buffers
+    # under AddressSanitizer where the compiler has it (operands, results and the parked tile are heap buffers), with
+    # misaligned vector accesses, indices out of a static array's bounds and out-of-range shifts ending the run as well
     exe = host_builds("asan") if host_builds.ok("asan") else host_builds("plain")
     rc, out, err = run_shares(exe)
-    assert "AddressSanitizer" not in err, err[:4000]
+    assert "AddressSanitizer" not in err and "runtime error" not in err, err[:4000]
     assert rc == 0, out[-2000:] + err[-2000:]
     lines = [l for l in out.splitlines() if "wrong of" in l]
     # 24 launches of the pipelined kernels x 2 load timings, 6 of the fused kernel, 9 tile numberings
@@ -226,7 +227,12 @@ class HostBuilds:
 
     def __init__(self, tmp):
         from concurrent.futures import ThreadPoolExecutor
-        jobs = {"asan": lambda: _build(tmp, "asan", extra=("-g", "-fsanitize=address")),
+        def checked():   # with the alignment, bounds and shift checks of UndefinedBehaviorSanitizer where its runtime is there
+            try:
+                return _build(tmp, "asan_ub", extra=("-g", "-fsanitize=address,alignment,bounds,shift", "-fno-sanitize-recover=all"))
+            except AssertionError:
+                return _build(tmp, "asan", extra=("-g", "-fsanitize=address"))
+        jobs = {"asan": checked,
                 "tsan": lambda: _build(tmp, "tsan", extra=("-g", "-fsanitize=thread")),
                 "tsan_broken": lambda: _build(tmp, "tsan_broken", _drop_barrier, extra=("-g", "-fsanitize=thread")),
                 "library": lambda: _build_library(tmp, "lib", drivers=("library_host.cpp", "library_cli.cpp"))}
