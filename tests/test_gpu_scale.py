@@ -143,19 +143,6 @@ def test_benchmark_table_rows():
         assert "|" in mp.format_row(r) and mp.HEADER.split("|")[0].strip() == "N_dim"
 
 
-def test_cutoff_table_rows():
-    """The cutoff table of main_profiling.py (classical kernel against Strassen levels, beside the rule of sthip_auto_levels) on
-    two small shapes: every column is there and timed, and the rule's column is what the library itself answers."""
-    import main_profiling as mp
-    import strassen_hip
-    rows = mp.profile_cutoff(torch.bfloat16, [(1024, 1024, 1024), (2048, 1024, 512)], max_levels=2, b_transposed=True, runs=4)
-    assert [(r["M"], r["N"], r["K"]) for r in rows] == [(1024, 1024, 1024), (2048, 1024, 512)]
-    for r in rows:
-        assert len(r["level_ms"]) == 3 and all(t > 0 for t in r["level_ms"]) and r["std_ms"] > 0
-        assert r["best_levels"] in (0, 1, 2)
-        assert r["rule_levels"] == strassen_hip.auto_levels(r["M"], r["N"], r["K"], torch.bfloat16, 2)
-
-
 def test_block_demo_forward_and_backward():
     """The decoder-block demo (reference train.py:322-350 on model/model.py:4-32): all four Linear
     layers are replaced and the block's output and weight gradients stay inside the bf16 bound."""
@@ -220,3 +207,16 @@ def test_kept_weight_sums_under_inference_mode():
         plain.weight.copy_(lin.weight)
         x = _gauss((1024, 1024), 141, 1.0, torch.bfloat16).cuda()
         assert torch.equal(lin(x), plain(x))
+
+
+def test_cutoff_table_rows():
+    """The cutoff table of main_profiling.py (classical kernel against Strassen levels, beside the rule of sthip_auto_levels) on
+    two small shapes: every column is there and timed, and the rule's column is what the library itself answers."""
+    import main_profiling as mp
+    import strassen_hip
+    rows = mp.profile_cutoff(torch.bfloat16, [(1024, 1024, 1024), (2048, 1024, 512)], max_levels=2, b_transposed=True, runs=4)
+    assert [(r["M"], r["N"], r["K"]) for r in rows] == [(1024, 1024, 1024), (2048, 1024, 512)]
+    for r in rows:
+        assert len(r["level_ms"]) == 3 and all(t > 0 for t in r["level_ms"]) and r["std_ms"] > 0
+        assert r["best_levels"] in (0, 1, 2)
+        assert r["rule_levels"] == strassen_hip.auto_levels(r["M"], r["N"], r["K"], torch.bfloat16, 2)
