@@ -15,120 +15,15 @@ k-step's barrier, one that moves the loader's cursor before the last load of a s
 kernel that waits one load short.
 """
 import os
-import re
-import shutil
 import subprocess
+import sys
 
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-CSRC = os.path.join(ROOT, "strassen-triton_amd", "csrc")
-MODEL = os.path.join(ROOT, "tests", "host_model")
-HEADERS = ("sthip_kernel.hpp", "sthip_kernel2.hpp", "sthip_kernel3.hpp", "sthip_kernel4.hpp", "sthip_kernel6.hpp")
-
-
-def _clang():
-    for cand in (os.environ.get("STHIP_HOST_CXX"), "/opt/rocm/lib/llvm/bin/clang++", shutil.which("clang++")):
-        if cand and os.path.exists(cand):
-            return cand
-    return None
-
-
-def strip_asm(text: str) -> str:
-    """Replaces every `asm volatile(...);` statement by an empty statement."""
-    out, i = [], 0
-    pat = re.compile(r"\basm\s+volatile\s*\(")
-    while True:
-        m = pat.search(text, i)
-        if not m:
-            out.append(text[i:])
-            return "".join(out)
-        out.append(text[i:m.start()])
-        j, depth, in_str = m.end(), 1, False
-        while depth:
-            c = text[j]
-            if in_str:
-                if c == "\\":
-                    j += 1
-                elif c == '"':
-                    in_str = False
-            elif c == '"':
-                in_str = True
-            elif c == "(":
-                depth += 1
-            elif c == ")":
-                depth -= 1
-            j += 1
-        k = j
-        while text[k] in " \t":
-            k += 1
-        assert text[k] == ";", text[m.start():k + 20]
-        out.append("((void)0);")
-        i = k + 1
-
-
-def _build(tmp, name, mutate=None, mutate_header="sthip_kernel4.hpp", extra=()):
-    inc = os.path.join(tmp, name)
-    os.makedirs(inc)
-    for h in HEADERS:
-        text = strip_asm(open(os.path.join(CSRC, h)).read()).replace("extern __shared__", "extern")
-        if mutate and h == mutate_header:
-            text = mutate(text)
-        open(os.path.join(inc, h), "w").write(text)
-    exe = os.path.join(inc, "kernel4_host")
-    cmd = [_clang(), "-std=c++17", "-O1", "-Wno-everything", "-no-pie", "-pthread", *extra, "-I", inc, "-I", MODEL,
-           "-I", os.path.join(ROOT, "include"), os.path.join(MODEL, "kernel4_host.cpp"), os.path.join(MODEL, "host_runtime.cpp"),
-           "-o", exe]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-3000:]
-    return exe
-
-
-def _build_library(tmp, name, extra=(), drivers=("library_host.cpp",)):
-    """Every translation unit of the library (strassen-triton_amd/build.py lists them) compiled for the host against the
-    stand-in HIP runtime of tests/host_model/hip/hip_runtime.h, linked with library_host.cpp and host_runtime.cpp."""
-    import glob
-    import importlib.util
-    from concurrent.futures import ThreadPoolExecutor
-    out = os.path.join(tmp, name)
-    os.makedirs(out)
-    for f in glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(CSRC, "*.hip")):
-        if os.path.basename(f) == "sthip_prims.hpp":   # the host build has its own (tests/host_model/sthip_prims.hpp)
-            continue
-        open(os.path.join(out, os.path.basename(f)), "w").write(strip_asm(open(f).read()).replace("extern __shared__", "extern"))
-    spec = importlib.util.spec_from_file_location("sthip_build", os.path.join(ROOT, "strassen-triton_amd", "build.py"))
-    build = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(build)
-    common = ["-std=c++17", "-O1", "-Wno-everything", "-pthread", *extra, "-I", MODEL, "-I", out, "-I", os.path.join(ROOT, "include")]
-
-    def compile_unit(unit):
-        obj, src, defs = unit
-        r = subprocess.run([_clang(), "-x", "c++", *common, *defs, "-c", os.path.join(out, src), "-o", os.path.join(out, obj)],
-                           capture_output=True, text=True)
-        assert r.returncode == 0, obj + "\n" + r.stderr[-3000:]
-        return os.path.join(out, obj)
-
-    with ThreadPoolExecutor(8) as pool:
-        objs = list(pool.map(compile_unit, build._units()))
-    runtime = os.path.join(out, "host_runtime.o")
-    r = subprocess.run([_clang(), *common, "-c", os.path.join(MODEL, "host_runtime.cpp"), "-o", runtime], capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-3000:]
-    exes = {}
-    for driver in drivers:
-        exes[driver] = os.path.join(out, driver[:-4])
-        r = subprocess.run([_clang(), *common, "-no-pie", os.path.join(MODEL, driver), runtime, *objs, "-o", exes[driver]],
-                           capture_output=True, text=True)
-        assert r.returncode == 0, r.stderr[-3000:]
-    return exes
-
-
-def run_shares(exe, shares=4, timeout=1800):
-    """The driver's cases dealt to `shares` processes that run side by side (a launch spends much of its time in barriers);
-    returns the worst exit code and everything printed."""
-    procs = [subprocess.Popen([exe, "%d/%d" % (i, shares)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True) for i in range(shares)]
-    outs = [p.communicate(timeout=timeout) for p in procs]
-    return max(abs(p.returncode) for p in procs), "".join(o[0] for o in outs), "".join(o[1] for o in outs)
-
+sys.path.insert(0, os.path.join(ROOT, "tests", "host_model"))
+import hostbuild  # noqa: E402
+from hostbuild import clang as _clang, strip_asm, run_shares, build_kernels as _build, build_library as _build_library  # noqa: E402,F401
 
 needs_clang = pytest.mark.skipif(_clang() is None, reason="no clang++ (the kernel headers use ext_vector_type)")
 
@@ -222,17 +117,41 @@ def test_broken_copies_are_caught(host_builds, name):
     assert "MODEL VIOLATION" in r.stderr or "FAILED" in r.stdout
 
 
+@needs_clang
+def test_preflight_gate_takes_the_kernel_directory_from_the_environment(tmp_path):
+    """tests/host_model/preflight.py is the one command a kernel source passes before it goes to a GPU.  Here it runs on a
+    directory that holds a copy of the committed 256 x 256 kernel header (kernel cases only: the library-level run is
+    test_library_through_its_c_abi_on_the_host), named through STHIP_KERNEL_DIR as a working copy would be."""
+    work = tmp_path / "variant"
+    work.mkdir()
+    (work / "sthip_kernel4.hpp").write_text(open(os.path.join(hostbuild.CSRC, "sthip_kernel4.hpp")).read())
+    env = dict(os.environ, STHIP_KERNEL_DIR=str(work))
+    r = subprocess.run([sys.executable, os.path.join(hostbuild.MODEL, "preflight.py"), "--no-library"], env=env,
+                       capture_output=True, text=True, timeout=1500)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "kernel sources from " + str(work) in r.stdout and "preflight: PASSED" in r.stdout
+
+
+@needs_clang
+def test_preflight_gate_refuses_a_broken_working_copy(tmp_path):
+    """The same command on a working copy with the mistake that once reached a GPU (the loader's cursor moved before the
+    step's last load, so that the last k-step reads past the operand) must fail."""
+    work = tmp_path / "variant"
+    work.mkdir()
+    (work / "sthip_kernel4.hpp").write_text(_advance_too_early(open(os.path.join(hostbuild.CSRC, "sthip_kernel4.hpp")).read()))
+    r = subprocess.run([sys.executable, os.path.join(hostbuild.MODEL, "preflight.py"), "--no-library", "--kernel-dir", str(work)],
+                       capture_output=True, text=True, timeout=1500)
+    assert r.returncode == 1, r.stdout[-3000:]
+    assert "preflight: FAILED" in r.stdout
+
+
 class HostBuilds:
     """Every host build these tests and tests/test_host_parity.py use, made side by side once per session."""
 
     def __init__(self, tmp):
         from concurrent.futures import ThreadPoolExecutor
-        def checked():   # with the alignment, bounds and shift checks of UndefinedBehaviorSanitizer where its runtime is there
-            try:
-                return _build(tmp, "asan_ub", extra=("-g", "-fsanitize=address,alignment,bounds,shift", "-fno-sanitize-recover=all"))
-            except AssertionError:
-                return _build(tmp, "asan", extra=("-g", "-fsanitize=address"))
-        jobs = {"asan": checked,
+        # "asan": with the alignment, bounds and shift checks of UndefinedBehaviorSanitizer where its runtime is there
+        jobs = {"asan": lambda: hostbuild.build_checked(tmp),
                 "tsan": lambda: _build(tmp, "tsan", extra=("-g", "-fsanitize=thread")),
                 "tsan_broken": lambda: _build(tmp, "tsan_broken", _drop_barrier, extra=("-g", "-fsanitize=thread")),
                 "library": lambda: _build_library(tmp, "lib", drivers=("library_host.cpp", "library_cli.cpp"))}
