@@ -201,3 +201,62 @@ def test_measured_cutoff_rule():
     assert lib.sthip_auto_levels(4096, 4096, 4096, f32, 3) == 0
     assert lib.sthip_auto_levels(768, 768, 8192, f32, 1) == 0
     assert lib.sthip_auto_levels(8192, 8192, 8192, bf16, 0) == 0 and lib.sthip_auto_levels(0, 8, 8, bf16, 1) == 0
+
+
+class _HostEvent:
+    """Stand-in for torch.cuda.Event on a machine without a GPU: wall-clock stamps."""
+
+    def __init__(self, enable_timing=False):
+        self.t = 0.0
+
+    def record(self):
+        import time
+        self.t = time.perf_counter()
+
+    def synchronize(self):
+        pass
+
+    def elapsed_time(self, other):
+        return (other.t - self.t) * 1e3 + 1e-3
+
+
+def test_cutoff_table_host_logic(monkeypatch, capsys):
+    """main_profiling.profile_cutoff with the GPU taken out: tensors on the CPU, host clock for events, and a stand-in for
+    strassen_hip.gemm that checks how it is called (positional out, `levels` / `algo` / `workspace` keywords, a workspace of
+    at least the size the library's own query returns).  What is left is the table's own logic: one classical column and
+    one per level, `best` = the fastest column, `rule` = the library's sthip_auto_levels (the real one, host arithmetic)."""
+    import main_profiling as mp
+    import strassen_hip
+    monkeypatch.setattr(torch.cuda, "Event", _HostEvent)
+    monkeypatch.setattr(torch.cuda, "empty_cache", lambda: None)
+    for name in ("randn", "empty"):
+        real = getattr(torch, name)
+        monkeypatch.setattr(torch, name, (lambda real: lambda *a, **k: real(*a, **{kk: v for kk, v in k.items() if kk != "device"}))(real))
+    calls = []
+
+    def gemm(a, b, out=None, *, algo="strassen", levels=1, workspace=None):
+        assert out is not None and out.shape == (a.shape[0], b.shape[1]) and out.dtype == a.dtype
+        lv = 0 if algo == "classic" else levels
+        need = strassen_hip.workspace_bytes(a, b, levels=lv) if lv else 0
+        assert algo in ("classic", "strassen") and (lv == 0 or (workspace is not None and workspace.numel() >= need))
+        calls.append((tuple(a.shape), tuple(b.shape), tuple(b.stride()), lv))
+        out.copy_(torch.matmul(a.float(), b.float()))
+        return out
+
+    monkeypatch.setattr(strassen_hip, "gemm", gemm)
+    rows = mp.profile_cutoff(torch.bfloat16, [(128, 128, 128), (256, 128, 64)], max_levels=2, b_transposed=True, runs=4)
+    assert [(r["M"], r["N"], r["K"]) for r in rows] == [(128, 128, 128), (256, 128, 64)]
+    for r in rows:
+        assert len(r["level_ms"]) == 3 and all(t > 0 for t in r["level_ms"]) and r["std_ms"] > 0
+        assert r["best_levels"] == min(range(3), key=lambda l: r["level_ms"][l])
+        assert r["rule_levels"] == strassen_hip.auto_levels(r["M"], r["N"], r["K"], torch.bfloat16, 2) == 0
+    assert {c[3] for c in calls} == {0, 1, 2}
+    assert all(c[2] == (1, c[1][0]) for c in calls)   # B is the transposed view of an N x K matrix
+    calls.clear()
+    rows = mp.profile_cutoff(torch.float32, [(128, 64, 128)], max_levels=3, runs=2)
+    assert len(rows[0]["level_ms"]) == 4 and {c[3] for c in calls} == {0, 1, 2, 3}
+    assert all(c[2] == (64, 1) for c in calls)
+    out = capsys.readouterr().out
+    assert out.count("M x N x K") == 2 and "128x64x128" in out and "3 level ms" in out
+    # the shapes --cutoff --max-n 32768 walks, and the level count it asks for
+    assert max(max(s) for s in mp._CUTOFF_SHAPES) == 32768 and all(len(s) == 3 for s in mp._CUTOFF_SHAPES)
