@@ -6,6 +6,8 @@
 #ifndef STRASSEN_HIP_DEBUG_H
 #define STRASSEN_HIP_DEBUG_H
 
+#include <stdint.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -25,6 +27,17 @@ int sthip_debug_transpose_read(void* out, void* stream);
  * With mask 2 the GEMM re-uses the sums a previous call left in the same workspace, so the
  * dominant kernel can be timed alone. */
 int sthip_debug_set_stages(int mask);
+
+/* After a call that ran as ONE launch (bit 4 above) with this workspace and these sizes: waits for
+ * `stream`, copies the launch's 16 dependency counters to counters[] (host memory; [0..2] finished
+ * units of the three sums jobs, [8..14] finished tiles of the seven products, [15] workgroups whose
+ * bounded wait for a producer expired) and returns counters[15], or a negative sthip_status.  The
+ * one-launch form never hangs, at the price that a workgroup which gives up goes on with whatever
+ * is in memory: when this returns anything but 0 the result of that call is undefined.  Its waits
+ * end only if workgroups start in blockIdx order, which the hardware does today and HIP does not
+ * promise; that, and being slower, is why the form stays behind a debug switch. */
+int sthip_debug_one_launch_counters(const void* workspace, int64_t M, int64_t N, int64_t K,
+                                    unsigned counters[16], void* stream);
 
 /* Overrides the tile table for later calls where the shape allows the forced tile: "128x128",
  * "256x128" (kernels that recombine in registers), "128x128g", "256x256" (grouped products),

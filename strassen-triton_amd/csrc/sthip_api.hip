@@ -2121,6 +2121,18 @@ int sthip_debug_force_tile(const char* tile) {
     return g_debug_tile.exchange(tile_code(tile));
 }
 
+int sthip_debug_one_launch_counters(const void* workspace, int64_t M, int64_t N, int64_t K, unsigned counters[16], void* stream) {
+    g_err[0] = 0;
+    if (!workspace || !counters || M <= 0 || N <= 0 || K <= 0 || M % 2 || N % 2 || K % 2)
+        return fail(STHIP_ERR_ARG, "one-launch counters: null pointer or sizes that no one-launch call takes");
+    hipError_t e = hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "hipStreamSynchronize failed: %s", hipGetErrorString(e));
+    const char* flags = reinterpret_cast<const char*>(workspace) + prepass_body_bytes(1, M / 2, N / 2, K / 2);
+    e = hipMemcpy(counters, flags, kFlagWords * sizeof(unsigned), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return fail(STHIP_ERR_HIP, "hipMemcpy of the counters failed: %s", hipGetErrorString(e));
+    return (int)std::min<unsigned>(counters[kFlagGaveUp], 1u << 30);
+}
+
 int sthip_debug_transpose_read(void* out, void* stream) {
     g_err[0] = 0;
     if (!out) return fail(STHIP_ERR_ARG, "null pointer");

@@ -158,6 +158,10 @@ hipError_t launch_fused5(const Fused5Params& p, int blocks, hipStream_t stream) 
     static OptIn opted;
     hipError_t e = opt_in_lds(opted, reinterpret_cast<const void*>(kern), kSmemBytes4);
     if (e != hipSuccess) return e;
+    // the tiles run the loader of the grouped kernel: the same bound on its 32-bit lane offsets
+    for (int s = 0; s < 7; ++s)
+        if (p.g.seg[s].a_ld >= (int64_t(1) << 26) || p.g.seg[s].b_ld >= (int64_t(1) << 26)) return hipErrorInvalidValue;
+    if (blocks <= 0 || p.tiles <= 0) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads4), kSmemBytes4, stream, p);
     return hipGetLastError();
 }

@@ -13,21 +13,25 @@ namespace sthip {
 // vmcnt(0); ordering is enforced by hand with wait_vmcnt() + the workgroup barrier.
 __device__ __forceinline__ void lds_dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
+                 :: "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
 }
 
 // lds_dma16 with the LDS address given as a uniform register plus a constant: one scalar instruction
 // for m0 and none for the global address (the rows of the load are part of the lane offset).
 __device__ __forceinline__ void lds_dma16_k(const void* sbase, uint32_t voff, uint32_t lds_addr, int k) {
     asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k) : "memory", "scc");
+                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k) : "memory", "scc", "m0");
 }
 // The same under a lane mask that is all ones or zero: with no lane enabled the load is not executed
-// (no memory access, nothing to wait for).  The caller runs with all lanes enabled.
+// (no memory access, nothing to wait for).  Contract: the caller runs with all 64 lanes enabled, and
+// the statement leaves them enabled; it is only called from the k-loop of gemm4p_kernel, whose
+// control flow depends on blockIdx and kernel arguments alone.  exec is deliberately not in the
+// clobber list: the statement restores the value the contract guarantees, and declaring it makes
+// the compiler fence every call with hazard nops and re-order the main loop around them.
 __device__ __forceinline__ void lds_dma16_km(const void* sbase, uint32_t voff, uint32_t lds_addr, int k, uint32_t mask) {
     asm volatile("s_mov_b32 exec_lo, %4\n\ts_mov_b32 exec_hi, %4\n\ts_add_u32 m0, %2, %3\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
-                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k), "s"(mask) : "memory", "scc");
+                 :: "s"(sbase), "v"(voff), "s"(lds_addr), "n"(k), "s"(mask) : "memory", "scc", "m0");
 }
 
 // The transposing LDS read (ds_read_b64_tr_b16): within each group of 16 lanes, lane r addresses four

@@ -36,6 +36,7 @@ SIGNATURES = {
     "sthip_debug_transpose_read": (_int, [_vp, _vp]),
     "sthip_debug_set_stages": (_int, [_int]),
     "sthip_debug_force_tile": (_int, [ctypes.c_char_p]),
+    "sthip_debug_one_launch_counters": (_int, [_vp, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_uint), _vp]),
 }
 
 _lib = None

@@ -5,6 +5,7 @@
 //   save NAME FILE            write a buffer to FILE
 //   units N                   compute units the "device" reports        tile NAME|-    force a tile of the pipelined paths
 //   stages MASK               sthip_debug_set_stages(MASK)
+//   one_launch_counters WS M N K TILES   sthip_debug_one_launch_counters: nobody gave up, every product counted TILES tiles
 //   expect CODE               the following call must return CODE (default 0)
 //   gemm / gemm_static / n_layers / run_accumulate / linear_strassen / linear / prepare / linear_prepared ARGS...
 //                             the entry point of include/strassen_hip.h of that name, arguments in its order, buffers by
@@ -113,6 +114,13 @@ int main(int argc, char** argv) {
             } else {
                 rc = sthip_gemm_static(A, B, C, batch, M, N, K, sA, sB, sC, dt, odt, algo, levels, acc, nullptr);
             }
+        } else if (op == "one_launch_counters") {
+            Buf* ws = buf(in);
+            const int64_t M = num(in), N = num(in), K = num(in), tiles = num(in);
+            unsigned c[16];
+            rc = sthip_debug_one_launch_counters(ws->p, M, N, K, c, nullptr);
+            for (int p = 8; p < 15 && rc == 0; ++p)
+                if (c[p] != (unsigned)tiles) { fprintf(stderr, "product %d counted %u tiles, expected %lld\n", p - 8, c[p], (long long)tiles); return 1; }
         } else if (op == "n_layers") {
             void *A = ptr(in), *B = ptr(in), *C = ptr(in);
             const int64_t n = num(in), ar = num(in), ac = num(in), br = num(in), bc = num(in);

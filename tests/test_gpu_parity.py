@@ -6,6 +6,7 @@ within the stated relative Frobenius tolerance on seeded Gaussian inputs:
     fp32            <= 1e-5
     bf16 / fp16     <= 2e-2   (fp32 accumulation and aggregation)
 """
+import ctypes
 import os
 
 import pytest
@@ -573,8 +574,10 @@ def test_one_level_as_one_launch_same_bits(hip, dtype, shape, tb):
             torch.cuda.synchronize()
         finally:
             lib.sthip_debug_set_stages(prev)
-        counters = ws[-256:].view(torch.int32)[:16].tolist()
-        assert counters[15] == 0, counters                       # nobody gave up
+        c16 = (ctypes.c_uint * 16)()
+        gave_up = lib.sthip_debug_one_launch_counters(ws.data_ptr(), M, N, K, c16, torch.cuda.current_stream().cuda_stream)   # waits for the stream
+        counters = list(c16)
+        assert gave_up == 0 and counters[15] == 0, counters      # nobody gave up
         assert counters[8:15] == [(M // 512) * (N // 512)] * 7   # the one-launch form did run: every tile counted
         assert torch.equal(got, want), rep
         A = (A * -0.5 + 0.125).to(dtype)

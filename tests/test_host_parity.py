@@ -275,8 +275,11 @@ def test_other_launch_forms_give_the_same_bits(cli, stages):
         sc = Script(cli)
         sc.add("tile", "256x256")
         sc.add("stages", mask)
+        ws = sc.workspace(1, 512, 512, 256, DT[BF], DT[BF], 1, 1)
         sc.add("gemm", sc.buf(A), sc.buf(B), sc.buf(C, back=True), 1, 512, 512, 256, *_strides3(A), *_strides3(B), *_strides3(C),
-               DT[BF], DT[BF], 1, 1, 0, sc.workspace(1, 512, 512, 256, DT[BF], DT[BF], 1, 1))
+               DT[BF], DT[BF], 1, 1, 0, ws)
+        if mask & 16:   # the debug query: no workgroup gave up waiting, each product counted its one tile
+            sc.add("one_launch_counters", ws, 512, 512, 256, 1)
         sc.run()
         outs.append(C)
     assert torch.equal(outs[0], outs[1])
