@@ -43,6 +43,22 @@ enum sthip_algo {
     STHIP_WINOGRAD = 2  /* 7 products, 15 add/sub (leaf level only; upper levels use Strassen) */
 };
 
+/* Optional, OR-ed into an `algo` argument: where a 16-bit problem of two or more levels rounds
+ * below its first level.  The reference's fp32-aggregating recursion rounds the first level's
+ * operand sums to base_dtype and recurses with base_dtype back at its default, fp32
+ * (fixed_strassen_fp32_agg.py:87-113), so everything deeper is fp32 arithmetic.
+ *   STHIP_SCHEDULE_REFERENCE  exactly that: first-level sums rounded to the operand type, then
+ *       widened; the seven half-size products run on the fp32 paths with levels - 1 levels
+ *       (fp32 matrix cores: 16 x slower than 16-bit ones).  Differs from the reference by fp32
+ *       summation order only.
+ *   STHIP_SCHEDULE_FAST       sums and products of every level rounded to the operand type, every
+ *       product on the 16-bit matrix cores.  Relative Frobenius distance from the reference in
+ *       bf16: 1.2e-2 at two levels, 2.3e-2 at three (fp16, with three more bits: below 5e-3).
+ * Neither flag: fast at two levels (the 49 products as one 16-bit launch), reference from three
+ * levels on, so that every default stays within 2e-2 of the reference.  fp32 problems and
+ * one-level calls ignore the flags.  Pass the same algo value to sthip_workspace_bytes. */
+enum sthip_schedule { STHIP_SCHEDULE_REFERENCE = 1 << 4, STHIP_SCHEDULE_FAST = 2 << 4 };
+
 /* General entry: C[b] (+)= A[b] x B[b] for b < batch, A is M x K, B is K x N, C is M x N.
  * stride*[3] = {batch, row, col} in elements; A and B need one unit stride among (row, col)
  * each (so NN / NT / TN / TT all work without copies; the other stride must stay below 2^26
@@ -145,7 +161,9 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
  * multiples take the kernels' edge tiles).  levels = 0 runs the classical product; levels < 0 runs
  * sthip_auto_levels(rows, out_features, in_features, dtype, -levels) levels, so that the layer never
  * takes a Strassen path that is slower than the library's classical kernel on that shape.
- * Workspace as sthip_workspace_bytes(1, rows, out, in, dtype, dtype, STHIP_STRASSEN, levels). */
+ * From three levels on (no counterpart: the reference's layers run one or two) every level rounds to the
+ * operand type, as with STHIP_SCHEDULE_FAST; sthip_linear_strassen_forward does the same.
+ * Workspace as sthip_workspace_bytes(1, rows, out, in, dtype, dtype, STHIP_STRASSEN | STHIP_SCHEDULE_FAST, levels). */
 int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y,
                          int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                          void* workspace, size_t workspace_bytes, void* stream);
@@ -154,8 +172,9 @@ int sthip_linear_forward(const void* x, const void* W, const void* bias, void* y
  * shape fastest on MI355X, from measurements of this library's own kernels against each other
  * (sweep of M, N, K in 768 .. 16384, both layouts of B).  16-bit: one level where the classical
  * product cannot fill the chip but the seven half-size products side by side can (at most 128
- * output tiles of 128 x 128 and k >= 4096: weight gradients), and from about 16384^3 up; a second
- * level from 32768^3, a third from 65536^3.  fp32: one level from 5e11 flop (8192 x 8192 x 4096), two
+ * output tiles of 128 x 128 and k >= 4096: weight gradients), and from 20480^3 up (at 16384^3 a level
+ * and the classical kernel are within 2 % of each other); a second level from 32768^3; never a
+ * third, which by default runs its inner products in fp32 (STHIP_SCHEDULE_REFERENCE).  fp32: one level from 5e11 flop (8192 x 8192 x 4096), two
  * from 1e12 (8192^3), three from 32768^3, and one level for products too small for the large-tile
  * kernel.  sthip_linear_forward applies this rule when its `levels` argument is negative.  No
  * counterpart in the reference, whose only cutoff is the min_size of replace_linear_with_strassen

@@ -480,7 +480,22 @@ struct Call {
     int force_tile = 0;
     BiasEpilogue bias;
     PreparedSums prep;
+    int sched = 0;   // kSchedAuto / kSchedReference / kSchedFast (bits 4-5 of the algo argument)
 };
+
+// Where 16-bit problems round below the first level.  The reference's fp32-aggregating recursion
+// rounds the first level's operand sums to base_dtype and then recurses with base_dtype left at
+// its default, fp32 (fixed_strassen_fp32_agg.py:99-113): every deeper sum, product and
+// recombination is fp32 arithmetic.  "Reference" does that: the first level's sums are rounded to
+// the operand type, widened to fp32, and the seven half-size products run on the fp32 paths with
+// levels - 1 levels.  "Fast" rounds the sums and products of every level to the operand type so
+// that every product runs on the 16-bit matrix cores (about 1.2e-2 from the reference at two
+// levels, 2.3e-2 at three in bf16).  Automatic: fast at two levels (all 49 products in one 16-bit
+// launch), reference from three levels on.
+enum { kSchedAuto = 0, kSchedReference = 1, kSchedFast = 2 };
+static bool reference_schedule(int dt, int levels, int sched) {
+    return dt != STHIP_F32 && levels >= 2 && (sched == kSchedReference || (sched == kSchedAuto && levels >= 3));
+}
 
 static const void* take_bias(Call& cx, const void* C, bool accumulate, bool out_f32) {
     if (!cx.bias.bias || C != cx.bias.target || accumulate || out_f32) return nullptr;
@@ -1158,7 +1173,8 @@ template <> __device__ __forceinline__ void st_elem<f16_t>(char* p, int64_t i, f
 // dst[rows x cols] (dense) = X[block a] + sign * X[block b], each block clipped to the
 // logical extent (lim_r, lim_c) of X and read as zero outside it.  sign = 0: copy block a.
 // The sum is formed in fp32 and rounded once (fixed_strassen_fp32_agg.py:87-96).
-template <class T>
+// TO = float with a 16-bit T: the sum is rounded to T all the same and stored widened, exactly.
+template <class T, class TO = T>
 __global__ void block_sum_kernel(char* dst, const char* X, int64_t rs, int64_t cs,
                                  int ra, int ca, int rb, int cb, int sign,
                                  int rows, int cols, int lim_r, int lim_c) {
@@ -1171,7 +1187,8 @@ __global__ void block_sum_kernel(char* dst, const char* X, int64_t rs, int64_t c
         const float w = ld_elem<T>(X, (int64_t)(rb + i) * rs + (int64_t)(cb + j) * cs);
         v = sign > 0 ? v + w : v - w;
     }
-    st_elem<T>(dst, idx, v);
+    if constexpr (__is_same(T, TO)) st_elem<T>(dst, idx, v);
+    else st_elem<TO>(dst, idx, round16<T>(v));
 }
 
 // C blocks from the seven products (dense fp32, mh x nh each):
@@ -1543,6 +1560,18 @@ static int block_sum(int dt, char* dst, View X, int ra, int ca, int rb, int cb, 
     return check_launch("block_sum");
 }
 
+// block_sum for a 16-bit X with the result stored as fp32 (the operands of the reference schedule's inner products).
+static int block_sum_widened(int dt, char* dst, View X, int ra, int ca, int rb, int cb, int sign,
+                             int64_t rows, int64_t cols, int64_t lim_r, int64_t lim_c, hipStream_t s) {
+    const int64_t n = rows * cols;
+    if (n == 0) return STHIP_OK;
+    const unsigned blocks = (unsigned)ceil_div(n, 256);
+#define GO(T) hipLaunchKernelGGL((block_sum_kernel<T, float>), dim3(blocks), dim3(256), 0, s, dst, X.p, X.rs, X.cs, ra, ca, rb, cb, sign, (int)rows, (int)cols, (int)lim_r, (int)lim_c)
+    if (dt == STHIP_F16) GO(f16_t); else GO(bf16_t);
+#undef GO
+    return check_launch("block_sum (widened)");
+}
+
 static int recombine(int out_dt, char* C, int64_t c_rs, int64_t c_cs, const float* Mbuf, int64_t mstride,
                      int64_t mh, int64_t nh, int64_t M, int64_t N, bool accumulate, hipStream_t s) {
     const int64_t n = mh * nh;
@@ -1674,9 +1703,12 @@ static int one_level_f32_grouped(View A, View B, char* C, int64_t c_rs, int64_t 
 
 // inner: the product is one of the seven of an upper level, which takes it in fp32 (16-bit operands
 // then keep their seven products in fp32 too: twice the room).
-static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels, bool inner = false) {
+static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int levels, bool inner = false, int sched = kSchedAuto) {
     const int64_t mh = Mp / 2, nh = Np / 2, kh = Kp / 2;
     if (levels <= 0) return 0;
+    if (reference_schedule(dt, levels, sched))   // one widened operand pair, seven fp32 products, the fp32 child
+        return align256(mh * kh * 4) + align256(kh * nh * 4) + 7 * align256(mh * nh * 4) +
+               workspace_for(mh, nh, kh, STHIP_F32, levels - 1, true);
     if (levels == 1) {
         if (fast_shape(dt, mh, nh, kh)) return prepass_bytes(1, mh, nh, kh, inner ? 4 : 2);
         if (dt == STHIP_F32 && mh > 0 && nh > 0 && kh > 0 && mh % kBM == 0 && nh % kBN == 0 && kh % 32 == 0)
@@ -1685,7 +1717,7 @@ static size_t workspace_for(int64_t Mp, int64_t Np, int64_t Kp, int dt, int leve
     }
     const size_t es = elem_size(dt);
     const size_t recursive = 5 * (align256(mh * kh * es) + align256(kh * nh * es)) + 7 * align256(mh * nh * 4) +
-                             workspace_for(mh, nh, kh, dt, levels - 1, true);
+                             workspace_for(mh, nh, kh, dt, levels - 1, true, sched);
     // two levels may run as one 49-product launch (two_level_flat) or, if the call's layout or
     // result type rules that out, as the host recursion: room for either
     if (levels == 2 && two_level_shape(dt, mh, nh, kh)) return std::max(recursive, two_level_bytes(mh, nh, kh));
@@ -1711,6 +1743,32 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
                             ws, ws_bytes, cx);
 
     const size_t es = elem_size(dt);
+    if (reference_schedule(dt, levels, cx.sched)) {
+        // fixed_strassen_fp32_agg.py:87-113: S1..S10 rounded to the operand type, everything below in fp32
+        const size_t a_b = align256(mh * kh * 4), b_b = align256(kh * nh * 4), m_b = align256(mh * nh * 4);
+        const size_t need = a_b + b_b + 7 * m_b;
+        if (!ws || ws_bytes < need) return fail(STHIP_ERR_WORKSPACE, "workspace too small: %zu < %zu", ws_bytes, need);
+        char* A32 = ws;
+        char* B32 = ws + a_b;
+        char* Mbuf = ws + a_b + b_b;
+        char* child_ws = ws + need;
+        const size_t child_bytes = std::min(ws_bytes - need, workspace_for(mh, nh, kh, STHIP_F32, levels - 1, true));
+        for (int q = 0; q < 7; ++q) {
+            const Term ta = kATerms[q], tb = kBTerms[q];
+            int rc = block_sum_widened(dt, A32, A, (ta.a >> 1) * (int)mh, (ta.a & 1) * (int)kh, (ta.b >> 1) * (int)mh, (ta.b & 1) * (int)kh,
+                                       ta.sign, mh, kh, M, K, cx.stream);
+            if (rc) return rc;
+            rc = block_sum_widened(dt, B32, B, (tb.a >> 1) * (int)kh, (tb.a & 1) * (int)nh, (tb.b >> 1) * (int)kh, (tb.b & 1) * (int)nh,
+                                   tb.sign, kh, nh, K, N, cx.stream);
+            if (rc) return rc;
+            Call child;
+            child.stream = cx.stream; child.stages = cx.stages; child.force_tile = cx.force_tile; child.sched = cx.sched;
+            rc = multiply(View{A32, kh, 1}, View{B32, nh, 1}, Mbuf + q * m_b, nh, 1, mh, nh, kh, mh, nh, kh, STHIP_F32, STHIP_F32,
+                          algo, levels - 1, false, child_ws, child_bytes, child, true);
+            if (rc) return rc;
+        }
+        return recombine(out_dt, C, c_rs, c_cs, reinterpret_cast<const float*>(Mbuf), (int64_t)(m_b / 4), mh, nh, M, N, accumulate, cx.stream);
+    }
     if (levels == 2 && (cx.stages & 8) && two_level_shape(dt, mh, nh, kh) && (!out_f32 || inner) && M == Mp && N == Np && K == Kp &&
         c_cs == 1 && c_rs % 8 == 0 && aligned_to(C, 16) && combos_ok(A, mh, kh) && combos_ok(B, kh, nh) &&
         (A.cs == 1 || A.rs == 1) && (B.cs == 1 || B.rs == 1) && ws && aligned_to(ws, 256) &&
@@ -1734,7 +1792,7 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
     char* child_ws = ws + need;
     // exactly what the query reserves for a child, however much more the caller passed: the kernels a
     // child picks depend on the room it is given
-    const size_t child_bytes = std::min(ws_bytes - need, workspace_for(mh, nh, kh, dt, levels - 1, true));
+    const size_t child_bytes = std::min(ws_bytes - need, workspace_for(mh, nh, kh, dt, levels - 1, true, cx.sched));
     // B-side sums of this level and of the levels below formed ahead of the call: read, never written
     const char* ready = vec && es == 2 && algo == STHIP_STRASSEN && levels >= 3 && B.rs == 1
                             ? take_prepared(cx, B.p, levels, kh, nh, prepared_bytes(levels, kh, nh)) : nullptr;
@@ -1784,7 +1842,7 @@ static int multiply(View A, View B, char* C, int64_t c_rs, int64_t c_cs,
         }
         // the child writes an fp32 product, never the caller's C: no bias for it, and only the sums of its own B operand
         Call child;
-        child.stream = cx.stream; child.stages = cx.stages; child.force_tile = cx.force_tile;
+        child.stream = cx.stream; child.stages = cx.stages; child.force_tile = cx.force_tile; child.sched = cx.sched;
         if (ready) {
             child.prep.sums = ready + 5 * sb_b + (size_t)q * child_prep; child.prep.bytes = child_prep; child.prep.target = b.p;
             child.prep.levels = levels - 1; child.prep.kh = kh / 2; child.prep.nh = nh / 2;
@@ -1801,7 +1859,7 @@ static int check_common(const void* A, const void* B, const void* C, int64_t bat
     if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(STHIP_ERR_SHAPE, "negative size");
     if (in_dt < 0 || in_dt > 2 || out_dt < 0 || out_dt > 2) return fail(STHIP_ERR_DTYPE, "unknown dtype (%d, %d)", in_dt, out_dt);
     if (out_dt != in_dt && out_dt != STHIP_F32) return fail(STHIP_ERR_DTYPE, "out dtype must equal in dtype or be fp32");
-    if (algo < 0 || algo > 2) return fail(STHIP_ERR_ARG, "unknown algo %d", algo);
+    if (algo < 0 || (algo & 15) > 2 || (algo >> 4) > 2) return fail(STHIP_ERR_ARG, "unknown algo %d", algo);
     if (levels < 0 || levels > 8) return fail(STHIP_ERR_ARG, "levels must be in [0, 8], got %d", levels);
     if (batch > 0 && M > 0 && N > 0 && (!C || (K > 0 && (!A || !B)))) return fail(STHIP_ERR_ARG, "null pointer");
     return STHIP_OK;
@@ -1850,6 +1908,8 @@ static int gemm_impl(Call& cx, const void* A, const void* B, void* C, int64_t ba
                      void* workspace, size_t workspace_bytes) {
     int rc = check_common(A, B, C, batch, M, N, K, in_dtype, out_dtype, algo, levels);
     if (rc) return rc;
+    if (algo >> 4) cx.sched = algo >> 4;   // STHIP_SCHEDULE_REFERENCE / STHIP_SCHEDULE_FAST
+    algo &= 15;
     if (!sA || !sB || !sC) return fail(STHIP_ERR_ARG, "null stride array");
     if (batch == 0 || M == 0 || N == 0) return STHIP_OK;
     const int es = elem_size(in_dtype), ces = elem_size(out_dtype);
@@ -1911,10 +1971,12 @@ static int auto_levels(int64_t M, int64_t N, int64_t K, int dt, int max_levels) 
         // classical
     } else {
         // 16-bit: the passes of a level cost about 14 n^2 bytes against n^3 / 4 flop saved: break-even
-        // near 16384^3 (1.02 - 1.05 x there, 0.92 x at 8192^3); a second level from 32768^3, a third from 65536^3
-        if (smallest >= 16384 || (smallest >= 8192 && K >= 16384 && M * N >= (int64_t)8192 * 16384)) levels = 1;
+        // near 16384^3 (0.92 x at 8192^3).  At 16384^3 a level measured 1.02 - 1.05 x before the classical
+        // kernel's main loop gained 4 % and a Strassen call 1.3 %: within 2 % either way since, so the rule
+        // waits for 20480; a second level from 32768^3.  Never a third: from three levels on the default
+        // schedule runs the inner products in fp32 as the reference does, which is not a speed-up.
+        if (smallest >= 20480 || (smallest >= 8192 && K >= 20480 && M * N >= (int64_t)8192 * 16384)) levels = 1;
         if (smallest >= 32768) levels = 2;
-        if (smallest >= 65536) levels = 3;
         // at most 128 output tiles of 128 x 128 and a long k (weight gradients): one classical product
         // leaves most CUs idle, seven half-size ones side by side do not (1.1 - 1.5 x from k = 4096)
         if (levels == 0 && ceil_div(M, 128) * ceil_div(N, 128) <= 128 && K >= 4096 &&
@@ -1927,6 +1989,9 @@ static int linear_forward_impl(Call& cx, const void* x, const void* W, const voi
                                int64_t rows, int64_t in_features, int64_t out_features, int dtype, int levels,
                                void* workspace, size_t workspace_bytes) {
     if (levels < 0) levels = auto_levels(rows, out_features, in_features, dtype, std::min(-levels, 8));
+    // the layers the reference has run one or two levels (model/layers.py:246); a third level and the weight-side
+    // sums kept for it are this library's own, and round at every level so that all products are 16-bit ones
+    cx.sched = kSchedFast;
     int rc = check_common(x, W, y, 1, rows, out_features, in_features, dtype, dtype, STHIP_STRASSEN, levels);
     if (rc) return rc;
     if (rows == 0 || out_features == 0) return STHIP_OK;
@@ -2012,6 +2077,9 @@ int sthip_gemm_static(const void* A, const void* B, void* C, int64_t batch, int6
 }
 
 size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, int algo, int levels) {
+    if (algo < 0 || (algo >> 4) > 2) return 0;
+    const int sched = algo >> 4;
+    algo &= 15;
     if (algo == STHIP_CLASSIC || levels <= 0 || M <= 0 || N <= 0 || K < 0 || levels > 8 || in_dtype < 0 || in_dtype > 2) return 0;
     const int64_t q = (int64_t)1 << levels;
     const int64_t Mp = round_up(M, q), Np = round_up(N, q), Kp = round_up(K, q);
@@ -2025,7 +2093,7 @@ size_t sthip_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int
             return prepass_bytes(batch, Mp / 2, Np / 2, Kp / 2, 4);
         return (size_t)batch * workspace_for(Mp, Np, Kp, in_dtype, 1);
     }
-    return workspace_for(Mp, Np, Kp, in_dtype, levels);
+    return workspace_for(Mp, Np, Kp, in_dtype, levels, false, sched);
 }
 
 int sthip_strassen_matmul_n_layers(const void* A, const void* B, void* C, int64_t n,
@@ -2049,6 +2117,7 @@ int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias
                                   int64_t rows, int64_t D, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream) {
     Call cx = begin_call(stream);
+    cx.sched = kSchedFast;   // as sthip_linear_forward
     int rc = check_common(x, W, y, 1, rows, D, D, dtype, dtype, STHIP_STRASSEN, levels);
     if (rc) return rc;
     if (levels < 1) return fail(STHIP_ERR_ARG, "levels must be >= 1, got %d", levels);

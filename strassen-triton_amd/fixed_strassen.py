@@ -33,12 +33,16 @@ def _strassen_base(A: Tensor, B: Tensor, base_dtype=torch.float32) -> Tensor:
 
 
 def strassen_matmul_n_layers(A: Tensor, B: Tensor, n_depth: int = 2, base_dtype=torch.float32) -> Tensor:
-    """n_depth-level Strassen product (reference fixed_strassen.py:59-126)."""
+    """n_depth-level Strassen product (reference fixed_strassen.py:59-126).  The reference does all
+    of its arithmetic in the input dtype at every level, so 16-bit inputs take the schedule that
+    rounds every level's operand sums and products to that dtype (sums and recombination are
+    still formed in fp32 and rounded once, which is closer to the exact product than the
+    reference's own additions in 16 bits)."""
     n = _check_square(A, B)
     levels = practical_levels(n, reference_levels(n, n_depth))
     if levels == 0:
         return strassen_hip.matmul(A, B, algo="classic", levels=0)
-    return strassen_hip.matmul(A, B, algo="strassen", levels=levels)
+    return strassen_hip.matmul(A, B, algo="strassen", levels=levels, schedule="fast")
 
 
 class _LinearFn(torch.autograd.Function):

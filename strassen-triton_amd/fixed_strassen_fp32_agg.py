@@ -29,8 +29,12 @@ def _strassen_base(A: Tensor, B: Tensor, base_dtype=torch.float32) -> Tensor:
 
 def strassen_matmul_n_layers(A: Tensor, B: Tensor, n_depth: int = 2, base_dtype=torch.float32) -> Tensor:
     """n_depth levels with fp32 aggregation (reference fixed_strassen_fp32_agg.py:58-125).
-    Every level's products run in base_dtype; the reference's inner calls fall back to fp32
-    products because they do not forward base_dtype (:99-113)."""
+    The reference's inner calls do not forward base_dtype (:99-113), so below the first level
+    it multiplies in fp32.  From three levels on this does the same (first-level sums rounded
+    to base_dtype, the seven half-size products on the fp32 kernels); at two levels all 49
+    quarter-size products run in base_dtype on the 16-bit matrix cores, 1.2e-2 from the
+    reference in bf16.  strassen_hip.gemm(..., schedule="reference") gives the reference's
+    schedule at two levels as well, schedule="fast" 16-bit products at every depth."""
     n = _check_square(A, B)
     A, B = A.to(base_dtype), B.to(base_dtype)
     levels = practical_levels(n, reference_levels(n, n_depth))

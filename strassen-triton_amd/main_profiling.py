@@ -203,8 +203,9 @@ def profile_cutoff(dtype=torch.bfloat16, shapes=None, max_levels: int = 2, b_tra
         r = dict(M=M, N=N, K=K, b_transposed=b_transposed, std_ms=_steady(lambda: torch.matmul(a, b, out=out), n))
         r["level_ms"] = [_steady(lambda: strassen_hip.gemm(a, b, out, algo="classic", levels=0), n)]
         for levels in range(1, max_levels + 1):
-            ws = torch.empty(max(1, strassen_hip.workspace_bytes(a, b, levels=levels)), dtype=torch.uint8, device="cuda")
-            r["level_ms"].append(_steady(lambda: strassen_hip.gemm(a, b, out, levels=levels, workspace=ws), n))
+            # "fast": every level on the 16-bit matrix cores (the default from three levels on runs its inner products in fp32)
+            ws = torch.empty(max(1, strassen_hip.workspace_bytes(a, b, levels=levels, schedule="fast")), dtype=torch.uint8, device="cuda")
+            r["level_ms"].append(_steady(lambda: strassen_hip.gemm(a, b, out, levels=levels, workspace=ws, schedule="fast"), n))
             del ws
         r["best_levels"] = min(range(max_levels + 1), key=lambda l: r["level_ms"][l])
         r["rule_levels"] = strassen_hip.auto_levels(M, N, K, dtype, max_levels)

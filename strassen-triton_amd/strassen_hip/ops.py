@@ -14,6 +14,20 @@ from . import _capi
 
 ALGO_CLASSIC, ALGO_STRASSEN, ALGO_WINOGRAD = 0, 1, 2
 _ALGOS = {"classic": ALGO_CLASSIC, "strassen": ALGO_STRASSEN, "winograd": ALGO_WINOGRAD}
+# OR-ed into the algo code (enum sthip_schedule): where 16-bit problems of two or more levels round below
+# the first level.  "reference": only the first level's sums, everything deeper in fp32 as the reference's
+# fp32-aggregating recursion does; "fast": every level, all products on the 16-bit matrix cores;
+# "auto": fast at two levels, reference from three.
+SCHEDULE_REFERENCE, SCHEDULE_FAST = 1 << 4, 2 << 4
+_SCHEDULES = {"auto": 0, "reference": SCHEDULE_REFERENCE, "fast": SCHEDULE_FAST}
+
+
+def _algo_code(algo, schedule: str = "auto") -> int:
+    code = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    try:
+        return code | _SCHEDULES[schedule]
+    except KeyError:
+        raise ValueError(f"schedule must be one of {sorted(_SCHEDULES)}, got {schedule!r}") from None
 _DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
@@ -59,10 +73,10 @@ def _workspace(nbytes: int, device) -> tuple[torch.Tensor | None, int]:
 
 
 def workspace_bytes(A: torch.Tensor, B: torch.Tensor, *, algo="strassen", levels: int = 1,
-                    out_dtype: torch.dtype | None = None) -> int:
+                    out_dtype: torch.dtype | None = None, schedule: str = "auto") -> int:
     """Bytes of scratch gemm(A, B, ...) would allocate; pass a uint8 tensor of at least that size
     as `workspace=` to re-use one allocation across calls."""
-    algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    algo = _algo_code(algo, schedule)
     batch = A.shape[0] if A.dim() == 3 else 1
     dt = _dtype_code(A.dtype)
     return _capi.load().sthip_workspace_bytes(batch, A.shape[-2], B.shape[-1], A.shape[-1], dt,
@@ -77,12 +91,13 @@ def auto_levels(M: int, N: int, K: int, dtype: torch.dtype, max_levels: int = 1)
 
 def gemm(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor | None = None, *, algo="strassen",
          levels: int = 1, accumulate: bool = False, out_dtype: torch.dtype | None = None,
-         workspace: torch.Tensor | None = None) -> torch.Tensor:
+         workspace: torch.Tensor | None = None, schedule: str = "auto") -> torch.Tensor:
     """out (+)= A @ B through sthip_gemm.  A: (b,) M x K, B: (b,) K x N, same dtype.
-    levels < 0: at most -levels levels, as many as the measured cutoff picks for the shape."""
+    levels < 0: at most -levels levels, as many as the measured cutoff picks for the shape.
+    schedule: "auto", "reference" or "fast" (see SCHEDULE_REFERENCE above)."""
     _require_gpu(A, B)
     lib = _capi.load()
-    algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    algo = _algo_code(algo, schedule)
     if levels < 0:
         levels = auto_levels(A.shape[-2], B.shape[-1], A.shape[-1], A.dtype, -levels)
         if levels == 0:
@@ -125,25 +140,26 @@ class StrassenMatmul(torch.autograd.Function):
     dA = dC @ B^T and dB = A^T @ dC read the saved operands through transposed views."""
 
     @staticmethod
-    def forward(ctx, A, B, algo, levels):
+    def forward(ctx, A, B, algo, levels, schedule="auto"):
         ctx.save_for_backward(A, B)
-        ctx.algo, ctx.levels = algo, levels
-        return gemm(A, B, algo=algo, levels=levels)
+        ctx.algo, ctx.levels, ctx.schedule = algo, levels, schedule
+        return gemm(A, B, algo=algo, levels=levels, schedule=schedule)
 
     @staticmethod
     def backward(ctx, dC):
         A, B = ctx.saved_tensors
         dC = dC.contiguous()
-        dA = gemm(dC, B.transpose(-1, -2), algo=ctx.algo, levels=ctx.levels) if ctx.needs_input_grad[0] else None
-        dB = gemm(A.transpose(-1, -2), dC, algo=ctx.algo, levels=ctx.levels) if ctx.needs_input_grad[1] else None
-        return dA, dB, None, None
+        kw = dict(algo=ctx.algo, levels=ctx.levels, schedule=ctx.schedule)
+        dA = gemm(dC, B.transpose(-1, -2), **kw) if ctx.needs_input_grad[0] else None
+        dB = gemm(A.transpose(-1, -2), dC, **kw) if ctx.needs_input_grad[1] else None
+        return dA, dB, None, None, None
 
 
-def matmul(A: torch.Tensor, B: torch.Tensor, algo="strassen", levels: int = 1) -> torch.Tensor:
+def matmul(A: torch.Tensor, B: torch.Tensor, algo="strassen", levels: int = 1, schedule: str = "auto") -> torch.Tensor:
     """Differentiable A @ B."""
     if torch.is_grad_enabled() and (A.requires_grad or B.requires_grad):
-        return StrassenMatmul.apply(A, B, algo, levels)
-    return gemm(A, B, algo=algo, levels=levels)
+        return StrassenMatmul.apply(A, B, algo, levels, schedule)
+    return gemm(A, B, algo=algo, levels=levels, schedule=schedule)
 
 
 def run_accumulate(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, *, algo="strassen", levels: int = 1,
@@ -180,7 +196,7 @@ def linear_forward(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor |
     x2d, weight = x2d.contiguous(), weight.contiguous()
     dt = _dtype_code(x2d.dtype)
     y = torch.empty((rows, D), dtype=x2d.dtype, device=x2d.device)
-    nbytes = lib.sthip_workspace_bytes(1, D, D, D, dt, dt, ALGO_STRASSEN, levels)
+    nbytes = lib.sthip_workspace_bytes(1, D, D, D, dt, dt, ALGO_STRASSEN | SCHEDULE_FAST, levels)
     ws, ws_ptr = _workspace(nbytes, x2d.device)
     b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
     with torch.cuda.device(x2d.device):
@@ -206,7 +222,7 @@ def linear_forward_any(x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tens
     if levels < 0:
         levels = lib.sthip_auto_levels(rows, d_out, d_in, dt, -levels)
     y = torch.empty((rows, d_out), dtype=x2d.dtype, device=x2d.device)
-    nbytes = lib.sthip_workspace_bytes(1, rows, d_out, d_in, dt, dt, ALGO_STRASSEN, levels)
+    nbytes = lib.sthip_workspace_bytes(1, rows, d_out, d_in, dt, dt, ALGO_STRASSEN | SCHEDULE_FAST, levels)
     ws, ws_ptr = _workspace(nbytes, x2d.device)
     b_ptr = bias.contiguous().data_ptr() if bias is not None else 0
     with torch.cuda.device(x2d.device):

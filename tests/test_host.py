@@ -92,10 +92,22 @@ def test_argument_errors_need_no_gpu():
     flat = lambda h: 10 * h * h * 2 + (70 + 49) * (h // 2) ** 2 * 2
     two = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 2)
     assert two == max(upper(512) + inner_sums(256), flat(512))
-    three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3)
+    # three levels, every level in the operand type (STHIP_SCHEDULE_FAST = 2 << 4 OR-ed into algo)
+    three = lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1 | (2 << 4), 3)
     assert three == upper(512) + max(upper(256) + inner_sums(128), flat(256))
     # fp32 never takes the one-launch form
-    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == 2 * 5 * 512 * 512 * 4 + 7 * 512 * 512 * 4 + f32(256)
+    f32_two = lambda h: 2 * 5 * h * h * 4 + 7 * h * h * 4 + f32(h // 2)
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1, 2) == f32_two(512)
+    # three levels by default, and two with STHIP_SCHEDULE_REFERENCE (1 << 4): one widened operand pair and seven fp32
+    # products of half size, then the fp32 problem of one level less
+    widened = lambda h: 2 * h * h * 4 + 7 * h * h * 4
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1, 3) == widened(512) + f32_two(256)
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1 | (1 << 4), 3) == widened(512) + f32_two(256)
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 1, 1, 1 | (1 << 4), 2) == widened(512) + f32(256)
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1 | (2 << 4), 2) == two            # two levels are fast by default
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 0, 0, 1 | (1 << 4), 2) == f32_two(512)   # fp32 ignores the flags
+    assert lib.sthip_workspace_bytes(1, 1024, 1024, 1024, 2, 2, 1 | (3 << 4), 2) == 0              # no such schedule
+    assert lib.sthip_gemm(one, one, one, 1, 64, 64, 64, big, big, big, 2, 2, 1 | (3 << 4), 2, 0, None, 0, None) == -5
 
 
 def test_weight_sums_size_and_argument_errors():
@@ -192,8 +204,10 @@ def test_measured_cutoff_rule():
     assert lib.sthip_auto_levels(2304, 768, 8192, bf16, 1) == 1
     assert lib.sthip_auto_levels(3072, 768, 8192, bf16, 1) == 0        # 144 output tiles: the classical kernel fills enough CUs
     assert lib.sthip_auto_levels(768, 768, 2048, bf16, 1) == 0         # k too short to pay for the passes
-    assert lib.sthip_auto_levels(16384, 16384, 16384, bf16, 3) == 1
+    assert lib.sthip_auto_levels(16384, 16384, 16384, bf16, 3) == 0    # within 2 % of the classical kernel either way
+    assert lib.sthip_auto_levels(20480, 20480, 20480, bf16, 3) == 1
     assert lib.sthip_auto_levels(32768, 32768, 32768, bf16, 3) == 2
+    assert lib.sthip_auto_levels(65536, 65536, 65536, bf16, 3) == 2    # a third 16-bit level would run in fp32 by default
     assert lib.sthip_auto_levels(32768, 32768, 32768, bf16, 1) == 1
     assert lib.sthip_auto_levels(8192, 8192, 8192, f32, 3) == 2 and lib.sthip_auto_levels(8192, 8192, 4096, f32, 3) == 1
     assert lib.sthip_auto_levels(2048, 4096, 2048, f32, 3) == 0      # the classical product on 64 x 64 tiles is faster
@@ -222,7 +236,7 @@ class _HostEvent:
 
 def test_cutoff_table_host_logic(monkeypatch, capsys):
     """main_profiling.profile_cutoff with the GPU taken out: tensors on the CPU, host clock for events, and a stand-in for
-    strassen_hip.gemm that checks how it is called (positional out, `levels` / `algo` / `workspace` keywords, a workspace of
+    strassen_hip.gemm that checks how it is called (positional out, `levels` / `algo` / `workspace` / `schedule` keywords, a workspace of
     at least the size the library's own query returns).  What is left is the table's own logic: one classical column and
     one per level, `best` = the fastest column, `rule` = the library's sthip_auto_levels (the real one, host arithmetic)."""
     import main_profiling as mp
@@ -234,10 +248,11 @@ def test_cutoff_table_host_logic(monkeypatch, capsys):
         monkeypatch.setattr(torch, name, (lambda real: lambda *a, **k: real(*a, **{kk: v for kk, v in k.items() if kk != "device"}))(real))
     calls = []
 
-    def gemm(a, b, out=None, *, algo="strassen", levels=1, workspace=None):
+    def gemm(a, b, out=None, *, algo="strassen", levels=1, workspace=None, schedule="auto"):
         assert out is not None and out.shape == (a.shape[0], b.shape[1]) and out.dtype == a.dtype
         lv = 0 if algo == "classic" else levels
-        need = strassen_hip.workspace_bytes(a, b, levels=lv) if lv else 0
+        assert lv == 0 or schedule == "fast"   # the table times 16-bit products at every level
+        need = strassen_hip.workspace_bytes(a, b, levels=lv, schedule=schedule) if lv else 0
         assert algo in ("classic", "strassen") and (lv == 0 or (workspace is not None and workspace.numel() >= need))
         calls.append((tuple(a.shape), tuple(b.shape), tuple(b.stride()), lv))
         out.copy_(torch.matmul(a.float(), b.float()))
