@@ -272,7 +272,7 @@ def test_three_levels_16bit(hip, dtype, tb, schedule):
     one-level figure: the undoubled bound.  schedule="fast": the top level keeps its seven
     products in fp32 and hands each to the 49-product 16-bit launch; every level rounds its operand
     sums to the operand type and the error about doubles per level (measured for bf16: 5.8e-3,
-    1.2e-2, 2.5e-2 for one, two, three levels), so that schedule is held to twice the bound."""
+    1.2e-2, 2.5e-2 for one, two, three levels), so that schedule is held to 1.5 x that figure."""
     A, B = _ints((1024, 512), 51, -1, 1, dtype), _ints((512, 1024), 52, -1, 1, dtype)
     C = hip.gemm(A.cuda(), _layout(B, tb), algo="strassen", levels=3, schedule=schedule)
     exact = A.double() @ B.double()
@@ -283,7 +283,8 @@ def test_three_levels_16bit(hip, dtype, tb, schedule):
     ref = Ag.double() @ Bg.double()
     rel = float(torch.linalg.norm(C.double() - ref) / torch.linalg.norm(ref))
     print(f"three levels {dtype} schedule {schedule}: {rel:.3e} from fp64")
-    assert rel <= (2 * TOL[dtype] if schedule == "fast" else TOL[dtype])
+    # fast: 1.5 x the 2.5e-2 measured for bf16; fp16 rounds eight times finer and stays inside the undoubled bound
+    assert rel <= (3.75e-2 if schedule == "fast" and dtype == torch.bfloat16 else TOL[dtype])
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])

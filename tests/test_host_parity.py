@@ -326,15 +326,16 @@ def test_two_levels_by_host_recursion(cli):
     assert torch.equal(C.double(), A.double() @ B.double())
 
 
-def _random_call(case):
+def _random_call(case, deep=False):
     """A seeded random sthip_gemm call: sizes aligned to tiles, to 8, or arbitrary; either layout of A and B; leading dimensions
     with padding; views that start 2 or 16 bytes into their storage; batch; fp32 or native result; accumulate; with and without
-    workspace; a forced tile; 1 .. 16 compute units."""
+    workspace; a forced tile; 1 .. 16 compute units.  deep: 16-bit operands, two or three levels, either rounding schedule
+    or the default."""
     import random
-    rnd = random.Random(1000 + case)
-    dt = rnd.choice([BF, BF, HF, SG])
-    algo = rnd.choice(["classic", "strassen", "strassen", "winograd"])
-    levels = 0 if algo == "classic" else rnd.choice([1, 1, 1, 2])
+    rnd = random.Random((5000 if deep else 1000) + case)
+    dt = rnd.choice([BF, HF] if deep else [BF, BF, HF, SG])
+    algo = rnd.choice(["strassen", "strassen", "winograd"] if deep else ["classic", "strassen", "strassen", "winograd"])
+    levels = rnd.choice([2, 3, 3]) if deep else 0 if algo == "classic" else rnd.choice([1, 1, 1, 2])
     kind = rnd.random()
     if kind < 0.35:
         M, N, K = (rnd.choice([64, 128]) * rnd.randint(1, 3) for _ in range(3))
@@ -347,6 +348,8 @@ def _random_call(case):
     batch = rnd.choice([0, 0, 0, 2])
     opts = dict(algo=algo, levels=levels, accumulate=rnd.random() < 0.3, workspace=rnd.random() < 0.8 or levels >= 2,
                 tile=rnd.choice([None, None, None, "128x128", "128x128g", "256x128", "256x256", "64x64"]), cus=rnd.choice([1, 2, 4, 8, 16]))
+    if deep:
+        opts["schedule"] = rnd.choice(["auto", "reference", "fast"])
     g = torch.Generator().manual_seed(case)
 
     def make(rows, cols, transposed, dtype, lo, hi):
@@ -369,6 +372,20 @@ def test_random_calls_exact(cli, case):
     host_gemm(cli, A, B, out=C, **opts)
     assert torch.equal(C.double(), A.double() @ B.double() + (C0.double() if opts["accumulate"] else 0)), opts
     after = C._base.clone()     # nothing outside the view of C (padding of its rows, the elements in front of it) was written
+    for whole in (around, after):
+        whole.as_strided(C.size(), C.stride(), C.storage_offset()).zero_()
+    assert torch.equal(around, after), opts
+
+
+@pytest.mark.parametrize("case", range(_grid(60, 6)))
+def test_random_deep_calls_exact(cli, case):
+    """The same for two and three levels of 16-bit operands on either rounding schedule (inner products in fp32, or every
+    level in the operand type) and on the default: small integers come out exact on all of them."""
+    A, B, C, opts = _random_call(case, deep=True)
+    C0, around = C.clone(), C._base.clone()
+    host_gemm(cli, A, B, out=C, **opts)
+    assert torch.equal(C.double(), A.double() @ B.double() + (C0.double() if opts["accumulate"] else 0)), opts
+    after = C._base.clone()
     for whole in (around, after):
         whole.as_strided(C.size(), C.stride(), C.storage_offset()).zero_()
     assert torch.equal(around, after), opts
