@@ -149,7 +149,8 @@ int sthip_run_accumulate(const void* A, const void* B, void* C,
  * the missing rows are simply never loaded or stored.  bias may be NULL; it is added to the
  * rounded product and the sum rounded again, as the reference's `+ bias` does -- inside the
  * recombination pass where the call runs as sums / grouped products / recombination, else by
- * a pass of its own. */
+ * a pass of its own.  Rounds at every level (see sthip_linear_forward); workspace as
+ * sthip_workspace_bytes(1, D, D, D, dtype, dtype, STHIP_STRASSEN | STHIP_SCHEDULE_FAST, levels). */
 int sthip_linear_strassen_forward(const void* x, const void* W, const void* bias, void* y,
                                   int64_t rows, int64_t D, int dtype, int levels,
                                   void* workspace, size_t workspace_bytes, void* stream);

@@ -456,7 +456,7 @@ def test_linear_strassen_forward_entry_point(cli, dtype, rows, D, levels, bias, 
     sc = Script(cli)
     sc.add("tile", tile or "-")
     sc.add("linear_strassen", sc.buf(x), sc.buf(W), sc.buf(b), sc.buf(y, back=True), rows, D, DT[dtype], levels,
-           sc.workspace(1, rows, D, D, DT[dtype], DT[dtype], 1, levels))
+           sc.workspace(1, rows, D, D, DT[dtype], DT[dtype], 1 | SCHEDULE["fast"], levels))
     sc.run()
     assert torch.equal(y.double(), x.double() @ W.double().t() + (b.double() if bias else 0))
 
@@ -473,7 +473,7 @@ def test_linear_forward_and_prepared_sums_same_bits(cli, dtype, levels, rows, d_
     ys = [torch.zeros(rows, d_out, dtype=dtype) for _ in range(3)]
     sc = Script(cli)
     bx, bw, bb = sc.buf(x), sc.buf(W), sc.buf(b)
-    ws = sc.workspace(1, rows, d_out, d_in, DT[dtype], DT[dtype], 1, abs(levels))
+    ws = sc.workspace(1, rows, d_out, d_in, DT[dtype], DT[dtype], 1 | SCHEDULE["fast"], abs(levels))   # as the header says for this entry
     sc.add("linear", bx, bw, bb, sc.buf(ys[0], back=True), rows, d_in, d_out, DT[dtype], levels, ws)
     if levels > 0:
         other = sc.buf(W.flip(0).contiguous())
