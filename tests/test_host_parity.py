@@ -219,11 +219,11 @@ def test_gaussian_against_the_oracle(cli, dtype, levels, shape, tile):
 
 # measured on the host build: 4.6e-5 (bf16, three levels), 1.8e-5 (fp16), 4.5e-5 (bf16, two levels, reference), 2.0e-2 (bf16,
 # three levels, fast), 9.2e-3 (bf16, two levels, fast)
-SCHEDULES = [(BF, 128, 3, "auto", 2e-4), (BF, 256, 3, "fast", 3e-2), (BF, 128, 2, "reference", 2e-4)]
+SCHEDULES = [(BF, 128, 3, "auto", 2e-4), (BF, 128, 2, "reference", 2e-4)]
 
 
-@pytest.mark.parametrize("dtype,n,depth,schedule,bound", _grid(SCHEDULES + [(HF, 256, 3, "auto", 1e-4), (BF, 256, 2, "auto", 2e-2)], SCHEDULES),
-                         ids=_name)
+@pytest.mark.parametrize("dtype,n,depth,schedule,bound",
+                         _grid(SCHEDULES + [(BF, 256, 3, "fast", 3e-2), (HF, 256, 3, "auto", 1e-4), (BF, 256, 2, "auto", 2e-2)], SCHEDULES), ids=_name)
 def test_cast_schedule_below_the_first_level(cli, dtype, n, depth, schedule, bound):
     """The reference rounds the first level's sums to base_dtype and runs everything deeper in fp32
     (fixed_strassen_fp32_agg.py:87-113; the oracle reproduces its outputs bit for bit, tests/test_golden_reference.py).
@@ -377,7 +377,7 @@ def test_random_calls_exact(cli, case):
     assert torch.equal(around, after), opts
 
 
-@pytest.mark.parametrize("case", range(_grid(60, 6)))
+@pytest.mark.parametrize("case", _grid(list(range(60)), [4]))   # twenty seconds and more each: the default run keeps one
 def test_random_deep_calls_exact(cli, case):
     """The same for two and three levels of 16-bit operands on either rounding schedule (inner products in fp32, or every
     level in the operand type) and on the default: small integers come out exact on all of them."""
@@ -422,7 +422,8 @@ def test_static_entry_point_refuses_what_does_not_fit(cli):
     sc.run()
 
 
-@pytest.mark.parametrize("dtype,n,levels", [(BF, 256, 1), (SG, 128, 2), (HF, 256, 2), (BF, 64, 3)], ids=_name)
+@pytest.mark.parametrize("dtype,n,levels", _grid([(BF, 256, 1), (SG, 128, 2), (HF, 256, 2), (BF, 64, 3)], [(BF, 256, 1), (SG, 128, 2), (HF, 256, 2)]),
+                         ids=_name)
 def test_n_layers_entry_point(cli, dtype, n, levels):
     """sthip_strassen_matmul_n_layers: square operands, B a transposed view (test_gpu_api.py:43)."""
     A, Bt = _ints((n, n), 61, -1, 1, dtype), _ints((n, n), 62, -1, 1, dtype)
