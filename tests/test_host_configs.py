@@ -1,0 +1,92 @@
+"""The five benchmark configurations at their REAL shapes on the CPU build of the library (tests/host_model/: the
+library's own sources compiled for the host, one host thread per lane), against the oracle at the configurations' bounds.
+What tests/test_gpu_parity.py checks on the card, checked where no card is at hand: the same seeded inputs, the same calls
+through the C ABI, the same kernels and path selection -- everything but the hardware's own execution.
+
+Minutes to hours each, so none of it runs unasked:
+
+    STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C4, C5, all
+
+Measured (8 host cores): C1 7.2e-7 from the oracle in 4 minutes; C5 attention projection forward 2.6e-5 and weight gradient
+6.9e-5 in 2 - 3 minutes each.  The figures of the other configurations are in the docstrings below as they were measured.
+"""
+import os
+
+import pytest
+import torch
+
+from oracle import strassen_oracle as O
+import test_host_parity
+from test_host_parity import BF, HF, SG, host_gemm, cli  # noqa: F401  (cli is the fixture that builds the driver)
+from test_kernel_host_model import _clang
+
+if os.environ.get("STHIP_HOST_CONFIGS"):
+    test_host_parity.Script.timeout = 8 * 3600
+
+ASKED = {c.strip() for c in os.environ.get("STHIP_HOST_CONFIGS", "").split(",") if c.strip()}
+pytestmark = pytest.mark.skipif(_clang() is None, reason="no clang++ for the host build")
+TOL = {SG: 1e-5, HF: 2e-2, BF: 2e-2}
+
+
+def _wanted(name):
+    return pytest.mark.skipif(not ({name, name[:2], "all"} & ASKED), reason="set STHIP_HOST_CONFIGS=%s (or all): minutes to hours on the host" % name)
+
+
+def _gauss(shape, seed, scale, dtype):
+    return (torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale).to(dtype)
+
+
+def _report(name, C, want, A, B, tol):
+    e_ref, e_exact = O.rel_fro(C.double(), want.double()), O.rel_fro(C.double(), A.double() @ B.double())
+    print(f"{name}: {e_ref:.3e} from the oracle, {e_exact:.3e} from fp64", flush=True)
+    assert e_ref <= tol and e_exact <= tol
+
+
+@_wanted("C1")
+def test_config1_fp32_one_level_1024(cli):  # noqa: F811
+    """1024^3 fp32, N(0,1), one level (fixed_strassen.py:11-57); on the card this is the 64 x 64 kernel with the sums formed
+    in the operand loads.  7.2e-7 from the oracle."""
+    A, B = _gauss((1024, 1024), 1234, 1.0, SG), _gauss((1024, 1024), 1235, 1.0, SG)
+    _report("config 1", host_gemm(cli, A, B, levels=1, cus=8), O.strassen_base(A, B), A, B, TOL[SG])
+
+
+@_wanted("C2")
+def test_config2_fp16_one_level_4096(cli):  # noqa: F811
+    """4096^3 fp16, N(0,1)/sqrt(K), one level with fp32 aggregation (fixed_strassen_fp32_agg.py:12-56): sums pass, seven
+    products on 256 x 256 tiles walked by the workgroups, recombination pass."""
+    n = 4096
+    A, B = _gauss((n, n), 1234, n ** -0.5, HF), _gauss((n, n), 1235, n ** -0.5, HF)
+    want = O.strassen_base_fp32_agg(A, B, HF, mm=O.mm_fp32_upcast)
+    _report("config 2", host_gemm(cli, A, B, levels=1, cus=16), want, A, B, TOL[HF])
+
+
+@pytest.mark.parametrize("depth", [pytest.param(1, marks=_wanted("C3a")), pytest.param(2, marks=_wanted("C3b"))])
+def test_config3_bf16_8192(cli, depth):  # noqa: F811
+    """8192^3 bf16, N(0,1)/sqrt(K): one level (the headline path) and two levels (49 products in one launch)."""
+    n = 8192
+    A, B = _gauss((n, n), 1234, n ** -0.5, BF), _gauss((n, n), 1235, n ** -0.5, BF)
+    want = O.strassen_matmul_n_layers(A, B, depth, BF, fp32_agg=True, mm=O.mm_fp32_upcast)
+    _report("config 3, %d level(s)" % depth, host_gemm(cli, A, B, levels=depth, cus=16), want, A, B, TOL[BF])
+
+
+@_wanted("C4")
+def test_config4_winograd_bf16(cli):  # noqa: F811
+    """Strassen-Winograd, 4096 x 8192 x 4096 bf16, U[-1,1]/sqrt(K): entry 0 of the configuration's batch of eight as a call of
+    its own (that batch entries do not influence each other is checked at small sizes, tests/test_host_parity.py)."""
+    b, M, K, N = 8, 4096, 8192, 4096
+    A = ((torch.rand((b, M, K), generator=torch.Generator().manual_seed(1234))[0] * 2 - 1) * K ** -0.5).to(BF)
+    B = ((torch.rand((b, K, N), generator=torch.Generator().manual_seed(1235))[0] * 2 - 1) * K ** -0.5).to(BF)
+    want = O.winograd_base(A, B, BF, fp32_agg=True, mm=O.mm_fp32_upcast)
+    _report("config 4, entry 0", host_gemm(cli, A, B, algo="winograd", levels=1, cus=16), want, A, B, TOL[BF])
+
+
+@_wanted("C5")
+@pytest.mark.parametrize("d_in,d_out", [(768, 768), (768, 2304), (768, 3072), (3072, 768), (768, 769)])
+def test_config5_gpt2_linears(cli, d_in, d_out):  # noqa: F811
+    """GPT-2-small Linear shapes, 8192 token rows, bf16 ~ N(0, 0.02), one level: forward x W^T (NT), input gradient dY W (NN),
+    weight gradient dY^T x (TN); 769 is the odd size that pads to even quadrants."""
+    rows = 8192
+    X, W, dY = _gauss((rows, d_in), 1234, 0.02, BF), _gauss((d_out, d_in), 1235, 0.02, BF), _gauss((rows, d_out), 1236, 0.02, BF)
+    for name, A, B in (("fwd", X, W.t()), ("dgrad", dY, W), ("wgrad", dY.t(), X)):
+        want = O.strassen_general(A, B, levels=1, base_dtype=BF, fp32_agg=True, mm=O.mm_fp32_upcast)
+        _report("config 5, %d -> %d %s" % (d_in, d_out, name), host_gemm(cli, A, B, levels=1, cus=16), want, A, B, TOL[BF])

@@ -56,6 +56,8 @@ class Script:
     """Statements for tests/host_model/library_cli.cpp: tensors become buffers of "device" memory (their whole storage, so
     views keep their strides), calls name them, results are read back into the tensors after run()."""
 
+    timeout = 900   # seconds for one run of the driver (tests/test_host_configs.py raises it)
+
     def __init__(self, cli):
         self.exe, self.tmp = cli
         self.lines, self.back, self.count = [], [], 0
@@ -90,7 +92,7 @@ class Script:
         path = os.path.join(self.tmp, "script.txt")
         with open(path, "w") as f:
             f.write("\n".join(self.lines) + "\n")
-        r = subprocess.run([self.exe, path], capture_output=True, text=True, timeout=900)
+        r = subprocess.run([self.exe, path], capture_output=True, text=True, timeout=self.timeout)
         assert r.returncode == 0, r.stderr[-2000:]
         for name, t in self.back:
             data = open(os.path.join(self.tmp, name + ".out"), "rb").read()
@@ -289,6 +291,19 @@ def test_paths_that_only_large_problems_take(cli, algo, levels, dtype, shape):
     else:
         C = host_gemm(cli, A, B, algo=algo, levels=levels, out_dtype=SG, cus=8, schedule="fast")
     assert torch.equal(C.double(), A.double() @ B.double())
+
+
+@pytest.mark.skipif(not FULL, reason="four minutes on the host: STHIP_HOST_FULL=1")
+def test_configuration_1_at_full_size(cli):
+    """One-level Strassen, 1024^3 fp32, N(0,1) from seeds 1234 / 1235 -- the first configuration at its real shape, on the kernel
+    it takes on the card (64 x 64 tiles, the quadrant sums formed in the operand loads) -- against the oracle's restatement of
+    fixed_strassen.py:11-57 at the configuration's bound.  Measured on the host build: 7.2e-7 (4.3e-7 from fp64)."""
+    n = 1024
+    A = torch.randn(n, n, generator=torch.Generator().manual_seed(1234))
+    B = torch.randn(n, n, generator=torch.Generator().manual_seed(1235))
+    C = host_gemm(cli, A, B, levels=1, cus=8)
+    assert O.rel_fro(C.double(), O.strassen_base(A, B).double()) <= 1e-5
+    assert O.rel_fro(C.double(), A.double() @ B.double()) <= 1e-5
 
 
 @pytest.mark.parametrize("stages", _grid([47, 31], [47]))
