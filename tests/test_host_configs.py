@@ -7,8 +7,10 @@ Minutes to hours each, so none of it runs unasked:
 
     STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C4, C5, all
 
-Measured (8 host cores): C1 7.2e-7 from the oracle in 4 minutes; C5 attention projection forward 2.6e-5 and weight gradient
-6.9e-5 in 2 - 3 minutes each.  The figures of the other configurations are in the docstrings below as they were measured.
+Measured (8 host cores; relative Frobenius distance from the oracle / from the fp64 product): C1 7.2e-7 / 4.3e-7 in 4
+minutes; C2 3.0e-5 / 7.2e-4 in 25 minutes (a GPU gave 3.1e-5 / 7.2e-4 on the same inputs); C4, entry 0, 9.2e-5 / 7.7e-3 in an
+hour; C5 between 3.3e-5 and 8.1e-5 from the oracle on the paths that round their products as the reference does and 4.0e-3
+on the kernels that keep them in fp32 (4.7e-3 from fp64 instead of 5.8e-3), two hours for the fifteen products.
 """
 import os
 
