@@ -5,12 +5,14 @@ through the C ABI, the same kernels and path selection -- everything but the har
 
 Minutes to hours each, so none of it runs unasked:
 
-    STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C4, C5, all
+    STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C3c (two at 4096^3), C4, C5, all
 
 Measured (8 host cores; relative Frobenius distance from the oracle / from the fp64 product): C1 7.2e-7 / 4.3e-7 in 4
 minutes; C2 3.0e-5 / 7.2e-4 in 25 minutes (a GPU gave 3.1e-5 / 7.2e-4 on the same inputs); C4, entry 0, 9.2e-5 / 7.7e-3 in an
 hour; C5 between 3.3e-5 and 8.1e-5 from the oracle on the paths that round their products as the reference does and 4.0e-3
-on the kernels that keep them in fp32 (4.7e-3 from fp64 instead of 5.8e-3), two hours for the fifteen products.
+on the kernels that keep them in fp32 (4.7e-3 from fp64 instead of 5.8e-3), two hours for the fifteen products; C3, one level,
+6.9e-5 / 5.8e-3 in three hours (a GPU: 8.5e-5 / 5.8e-3); two levels at 4096^3 1.13e-2 / 1.20e-2 in twenty minutes (a GPU at
+8192^3: 1.18e-2 / 1.24e-2).
 """
 import os
 
@@ -69,6 +71,16 @@ def test_config3_bf16_8192(cli, depth):  # noqa: F811
     A, B = _gauss((n, n), 1234, n ** -0.5, BF), _gauss((n, n), 1235, n ** -0.5, BF)
     want = O.strassen_matmul_n_layers(A, B, depth, BF, fp32_agg=True, mm=O.mm_fp32_upcast)
     _report("config 3, %d level(s)" % depth, host_gemm(cli, A, B, levels=depth, cus=16), want, A, B, TOL[BF])
+
+
+@_wanted("C3c")
+def test_two_levels_bf16_4096(cli):  # noqa: F811
+    """The two-level form of configuration 3 at an eighth of its work (4096^3; the 8192^3 run takes some thirteen core-hours
+    on the host): sums of both levels in one pass, the 49 quarter-size products as one launch, both recombinations in one pass."""
+    n = 4096
+    A, B = _gauss((n, n), 1234, n ** -0.5, BF), _gauss((n, n), 1235, n ** -0.5, BF)
+    want = O.strassen_matmul_n_layers(A, B, 2, BF, fp32_agg=True, mm=O.mm_fp32_upcast)
+    _report("two levels, 4096^3 bf16", host_gemm(cli, A, B, levels=2, cus=16), want, A, B, TOL[BF])
 
 
 @_wanted("C4")
