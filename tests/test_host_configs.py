@@ -5,7 +5,7 @@ through the C ABI, the same kernels and path selection -- everything but the har
 
 Minutes to hours each, so none of it runs unasked:
 
-    STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C3c (two at 4096^3), C4, C5, all
+    STHIP_HOST_CONFIGS=C1,C2 python -m pytest tests/test_host_configs.py -s     # or C3a (one level), C3b (two), C3c (two at 4096^3), C4, C5, L4 (LinearStrassen 4096), all
 
 Measured (8 host cores; relative Frobenius distance from the oracle / from the fp64 product): C1 7.2e-7 / 4.3e-7 in 4
 minutes; C2 3.0e-5 / 7.2e-4 in 25 minutes (a GPU gave 3.1e-5 / 7.2e-4 on the same inputs); C4, entry 0, 9.2e-5 / 7.7e-3 in an
@@ -21,7 +21,7 @@ import torch
 
 from oracle import strassen_oracle as O
 import test_host_parity
-from test_host_parity import BF, HF, SG, host_gemm, cli  # noqa: F401  (cli is the fixture that builds the driver)
+from test_host_parity import BF, DT, HF, SCHEDULE, SG, Script, host_gemm, cli  # noqa: F401  (cli is the fixture that builds the driver)
 from test_kernel_host_model import _clang
 
 if os.environ.get("STHIP_HOST_CONFIGS"):
@@ -104,3 +104,23 @@ def test_config5_gpt2_linears(cli, d_in, d_out):  # noqa: F811
     for name, A, B in (("fwd", X, W.t()), ("dgrad", dY, W), ("wgrad", dY.t(), X)):
         want = O.strassen_general(A, B, levels=1, base_dtype=BF, fp32_agg=True, mm=O.mm_fp32_upcast)
         _report("config 5, %d -> %d %s" % (d_in, d_out, name), host_gemm(cli, A, B, levels=1, cus=16), want, A, B, TOL[BF])
+
+
+@pytest.mark.parametrize("depth", [pytest.param(1, marks=_wanted("L4")), pytest.param(2, marks=_wanted("L4"))])
+def test_linear_strassen_4096(cli, depth):  # noqa: F811
+    """LinearStrassen(4096) with 1000 input rows, bias, bf16, depth 1 and 2 (sthip_linear_strassen_forward) against the oracle's
+    restatement of model/layers.py:246-274 -- pad to D x D, _strassen_base or the two-layer function of strassen.py (which adds in
+    bf16 at both levels, hence twice the bound at depth 2, as in tests/test_gpu_scale.py), slice, + bias."""
+    D, rows = 4096, 1000
+    w, b, x = _gauss((D, D), 107, D ** -0.5, BF), _gauss((D,), 108, 1.0, BF), _gauss((rows, D), 109, 1.0, BF)
+    y = torch.zeros(rows, D, dtype=BF)
+    sc = Script(cli)
+    sc.add("units", 16)
+    sc.add("linear_strassen", sc.buf(x), sc.buf(w), sc.buf(b), sc.buf(y, back=True), rows, D, DT[BF], depth,
+           sc.workspace(1, D, D, D, DT[BF], DT[BF], 1 | SCHEDULE["fast"], depth))
+    sc.run()
+    want = O.linear_strassen_forward(x, w, b, depth, mm=O.mm_fp32_upcast)
+    exact = x.double() @ w.double().t() + b.double()
+    err, err64, ora64 = O.rel_fro(y, want), O.rel_fro(y, exact), O.rel_fro(want, exact)
+    print(f"LinearStrassen 4096, {rows} rows, depth {depth}: {err:.3e} from the oracle, {err64:.3e} from fp64 (the oracle: {ora64:.3e})", flush=True)
+    assert err64 <= TOL[BF] and err <= TOL[BF] * depth and err64 <= ora64 * 1.05
