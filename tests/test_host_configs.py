@@ -12,7 +12,8 @@ minutes; C2 3.0e-5 / 7.2e-4 in 25 minutes (a GPU gave 3.1e-5 / 7.2e-4 on the sam
 hour; C5 between 3.3e-5 and 8.1e-5 from the oracle on the paths that round their products as the reference does and 4.0e-3
 on the kernels that keep them in fp32 (4.7e-3 from fp64 instead of 5.8e-3), two hours for the fifteen products; C3, one level,
 6.9e-5 / 5.8e-3 in three hours (a GPU: 8.5e-5 / 5.8e-3); two levels at 4096^3 1.13e-2 / 1.20e-2 in twenty minutes (a GPU at
-8192^3: 1.18e-2 / 1.24e-2).
+8192^3: 1.18e-2 / 1.24e-2); LinearStrassen(4096) on 1000 rows 3.1e-3 / 2.9e-3 at depth 1 and 4.7e-3 / 4.3e-3 at depth 2, whose
+oracle adds in bf16 and is itself 3.6e-3 and 5.8e-3 from fp64 (seventy minutes for the two).
 """
 import os
 
